@@ -1,0 +1,47 @@
+"""ctypes binding of libelmo_xmc.so (declarations: include/elmo_xmc.h).  There is no fallback: if the
+library has not been built, or a call fails, an exception is raised."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libelmo_xmc.so")
+
+ROUND_MODES = {"rtn": 0, "sr_philox": 1, "sr_fast": 2}
+
+_lib = None
+
+
+class XmcError(RuntimeError):
+    pass
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise XmcError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc --offload-arch=gfx950); there is no CPU fallback for the classifier step")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i32, f32, sz, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_longlong
+    lib.xmc_version.restype = i32
+    lib.xmc_error_string.restype = ctypes.c_char_p
+    lib.xmc_error_string.argtypes = [i32]
+    lib.xmc_workspace_bytes.restype = sz
+    lib.xmc_workspace_bytes.argtypes = [i32, i32]
+    lib.xmc_fp8_step.restype = i32
+    lib.xmc_fp8_step.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, vp, i32, f32,
+                                 ctypes.POINTER(ctypes.c_uint32), i32, f32, f32, vp, vp, vp, sz, vp]
+    lib.xmc_fp8_forward.restype = i32
+    lib.xmc_fp8_forward.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp, sz, vp]
+    lib.xmc_step_error_word.restype = i32
+    lib.xmc_step_error_word.argtypes = [vp, i32, i32, vp]
+    _lib = lib
+    return lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = load().xmc_error_string(status).decode()
+        raise XmcError(f"{what} failed: {msg} (status {status})")

@@ -1,0 +1,171 @@
+// extern "C" surface of libelmo_xmc.so: argument validation, workspace carving and kernel launches.
+// Declarations and the reference interfaces they replace: include/elmo_xmc.h.
+#include "../../include/elmo_xmc.h"
+#include "xmc_fp8_step.hip"
+
+using namespace xmc;
+
+namespace {
+
+struct DeviceInfo { int ok; int cus; };
+
+DeviceInfo device_info() {
+  static DeviceInfo cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DeviceInfo{-1, 0};
+  if (cached[dev].ok == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DeviceInfo{-1, 0};
+    cached[dev].cus = prop.multiProcessorCount;
+    cached[dev].ok = (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : -1;
+    // opt in to the full 160 KiB of LDS once per device
+    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
+    (void)hipFuncSetAttribute((const void*)sort_keys_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
+  }
+  return cached[dev];
+}
+
+inline bool aligned16(const void* q) { return ((uintptr_t)q & 15) == 0; }
+
+int check_common(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x, int batch, int features,
+                 const void* workspace, size_t workspace_bytes) {
+  if (!chunk_ptrs || !x || !workspace) return XMC_ERR_NULL;
+  if (features != D || batch <= 0 || batch > BP || batch % 16 != 0) return XMC_ERR_SHAPE;
+  if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return XMC_ERR_SHAPE;
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
+  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1) return XMC_ERR_RANGE;
+  for (int c = 0; c < num_chunks; c++) {
+    if (!chunk_ptrs[c]) return XMC_ERR_NULL;
+    if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
+  }
+  if (!aligned16(x) || ((uintptr_t)workspace & 255) != 0) return XMC_ERR_ALIGN;
+  if (workspace_bytes < xmc_workspace_bytes(num_chunks, rows_per_chunk)) return XMC_ERR_WORKSPACE;
+  return XMC_OK;
+}
+
+int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
+
+}  // namespace
+
+extern "C" {
+
+int xmc_version(void) { return 1; }
+
+const char* xmc_error_string(int status) {
+  switch (status) {
+    case XMC_OK: return "ok";
+    case XMC_ERR_NULL: return "null pointer";
+    case XMC_ERR_SHAPE: return "unsupported shape (features must be 768, batch a multiple of 16 and <= 128, rows per chunk a multiple of 16)";
+    case XMC_ERR_ALIGN: return "device pointer not sufficiently aligned";
+    case XMC_ERR_RANGE: return "too many chunks, labels or positives";
+    case XMC_ERR_WORKSPACE: return "workspace too small";
+    case XMC_ERR_MODE: return "unknown rounding mode";
+    case XMC_ERR_LAUNCH: return "kernel launch failed";
+    case XMC_ERR_DEVICE: return "current device is not a gfx950 GPU with at least 16 compute units";
+    default: return "unknown status";
+  }
+}
+
+size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk) {
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
+  size_t tiles = (size_t)num_chunks * ((rows_per_chunk + TL - 1) / TL);
+  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256;
+}
+
+int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                 int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                 float scale_w, float scale_x, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                 size_t workspace_bytes, void* stream_) {
+  int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
+  if (st != XMC_OK) return st;
+  if (!grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
+  if (nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
+  if (round_mode < XMC_ROUND_RTN || round_mode > XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
+  if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
+  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  DeviceInfo di = device_info();
+  if (di.ok != 1 || di.cus < 16) return XMC_ERR_DEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  unsigned char* ws = (unsigned char*)workspace;
+
+  const int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;   // one workgroup per CU, pairs on one XCD
+  const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
+  const int num_tiles = num_chunks * tiles_per_chunk;
+  int n_pad = 0;
+  if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
+
+  (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
+  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
+                                                              (unsigned short*)(ws + WS_XT));
+  if (n_pad > 0)
+    sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
+  tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
+                                                                tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
+  StepParams p;
+  for (int c = 0; c < MAX_CHUNKS; c++) {
+    p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
+    p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+  }
+  p.num_chunks = num_chunks;
+  p.rows_per_chunk = rows_per_chunk;
+  p.tiles_per_chunk = tiles_per_chunk;
+  p.num_tiles = num_tiles;
+  p.xq = ws + WS_XQ;
+  p.xt = (const bf16x8*)(ws + WS_XT);
+  p.keys = (const unsigned*)(ws + WS_KEYS);
+  p.tile_ptr = (const int*)(ws + WS_TILEPTR);
+  p.partial = (floatx4*)(ws + WS_PARTIAL);
+  p.flags = (int*)(ws + WS_FLAGS);
+  p.zscale = scale_w * scale_x;
+  p.lr_eff = lr / scale_w;
+  p.batch = batch;
+  switch (round_mode) {
+    case XMC_ROUND_RTN: fp8_step_kernel<ROUND_RTN><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+    case XMC_ROUND_SR_PHILOX: fp8_step_kernel<ROUND_SR_PHILOX><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+    default: fp8_step_kernel<ROUND_SR_FAST><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+  }
+  reduce_gx_kernel<<<96, NT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), grid, scale_w, grad_x_f32,
+                                         (unsigned short*)grad_x_bf16, batch);
+  return launch_status();
+}
+
+int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                    int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
+                    long long num_labels, void* workspace, size_t workspace_bytes, void* stream_) {
+  int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
+  if (st != XMC_OK) return st;
+  if (!out_bf16) return XMC_ERR_NULL;
+  if (num_labels <= 0 || out_stride < num_labels || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
+  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  unsigned char* ws = (unsigned char*)workspace;
+  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
+                                                              (unsigned short*)(ws + WS_XT));
+  const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
+  const int grid = tiles_per_chunk < 4 * di.cus ? tiles_per_chunk : 4 * di.cus;
+  for (int c = 0; c < num_chunks; c++)
+    fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
+                                                       scale_w * scale_x, (unsigned short*)out_bf16, out_stride,
+                                                       (long long)c * rows_per_chunk, num_labels, batch);
+  return launch_status();
+}
+
+int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream_) {
+  (void)num_chunks; (void)rows_per_chunk;
+  if (!workspace) return XMC_ERR_NULL;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  const int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;
+  int word = 0;
+  if (hipMemcpyAsync(&word, (const unsigned char*)workspace + WS_FLAGS + (size_t)grid * 4, 4, hipMemcpyDeviceToHost,
+                     (hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
+  return word;
+}
+
+}  // extern "C"

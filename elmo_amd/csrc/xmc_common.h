@@ -1,0 +1,111 @@
+// Shared device helpers and compile-time geometry for the gfx950 XMC classifier kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xmc {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// ---- geometry (one MI355X compute unit works on a 64-label tile; a pair of CUs shares a tile, each
+//      owning one half of the 768 input features for the two gradient GEMMs and the update)
+constexpr int D = 768;            // input features (row length of W, bytes per FP8 row)
+constexpr int BP = 128;           // padded batch rows
+constexpr int TL = 64;            // labels per tile
+constexpr int NT = 256;           // threads per workgroup (4 wavefronts of 64)
+constexpr int HALF = D / 2;       // features owned by one CU of a pair
+constexpr int WCOLS = HALF / 4;   // features owned by one wavefront (96)
+constexpr int WS = D + 16;        // LDS row stride of the W tile, bytes (49 x 16)
+constexpr int GT_S = TL * 2 + 16; // LDS row stride of G^T [b][l], bytes
+constexpr int GL_S = BP * 2 + 16; // LDS row stride of G   [l][b], bytes
+constexpr int WT_BYTES = TL * WS;
+constexpr int LDS_BYTES = 2 * WT_BYTES + BP * GT_S + TL * GL_S;
+constexpr int MAX_CHUNKS = 64;
+constexpr int MAX_POS = 16384;    // positives per step the single-workgroup sort handles
+
+// workspace layout (byte offsets), all 256-byte aligned
+constexpr int MAX_WG = 256;                                   // workgroups of the persistent step kernel
+constexpr size_t WS_XQ = 0;                                   // FP8 logits operands   BP*D
+constexpr size_t WS_XT = WS_XQ + (size_t)BP * D;              // bf16 grad_W operands  BP*D*2
+constexpr size_t WS_KEYS = WS_XT + (size_t)BP * D * 2;        // sorted positive keys  MAX_POS*4
+constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // pair counters + error word (4 KiB)
+constexpr size_t WS_PARTIAL = WS_FLAGS + 4096;                // MAX_WG * 48 * 256 * 16 bytes of grad_X partials
+constexpr size_t WS_TILEPTR = WS_PARTIAL + (size_t)MAX_WG * 48 * NT * 16;   // tile_ptr[num_tiles + 1]
+
+__device__ __forceinline__ float bf16_rt(float f) { return (float)(__bf16)f; }
+
+__device__ __forceinline__ unsigned short bf16_bits(float f) {
+  __bf16 b = (__bf16)f;
+  unsigned short u;
+  __builtin_memcpy(&u, &b, 2);
+  return u;
+}
+__device__ __forceinline__ float bf16_from_bits(unsigned short u) { return __uint_as_float((unsigned)u << 16); }
+
+__device__ __forceinline__ float clamp448(float t) { return __builtin_fminf(__builtin_fmaxf(t, -448.0f), 448.0f); }
+
+// Philox-4x32-10, counter (off,0,0,0), key (seed_lo, seed_hi); returns word 0.
+__device__ __forceinline__ unsigned philox_word0(unsigned off, unsigned k0, unsigned k1) {
+  unsigned c0 = off, c1 = 0, c2 = 0, c3 = 0;
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    unsigned hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    unsigned hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0; c1 = lo1; c2 = hi0 ^ c3 ^ k1; c3 = lo0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+// Counter hash of the fast stochastic-rounding mode: one 32-bit mix per 4 consecutive weights of a row,
+// expanded to four words by odd multipliers.  idx = global_row * (D/4) + col/4.
+__device__ __forceinline__ unsigned fast_mix(unsigned idx, unsigned seed) {
+  unsigned h = idx * 0x9E3779B1u + seed;
+  h ^= h >> 16; h *= 0x85EBCA77u; h ^= h >> 15;
+  return h;
+}
+__device__ __forceinline__ unsigned fast_word(unsigned h, int i) {
+  const unsigned k[4] = {0xC2B2AE3Du, 0x27D4EB2Fu, 0x165667B1u, 0x9E3779B1u};
+  return h * k[i];
+}
+
+enum RoundMode { ROUND_RTN = 0, ROUND_SR_PHILOX = 1, ROUND_SR_FAST = 2 };
+
+// Round four updated weights (fp32) of one row, columns col..col+3, to e4m3 codes packed in a dword.
+//   RTN        round to nearest even, saturating at +-448
+//   SR_PHILOX  bits(t) + (philox(seed, row*D+col) & 0xFFFFF), clear low 20 bits, then the RTN cast
+//   SR_FAST    true stochastic rounding on the e4m3 grid (subnormals included) by the hardware
+//              converter, random word from fast_mix/fast_word
+template <int MODE>
+__device__ __forceinline__ unsigned round4(float t0, float t1, float t2, float t3, unsigned row_in_chunk,
+                                           unsigned grow, unsigned col, unsigned seed) {
+  float t[4] = {t0, t1, t2, t3};
+  if (MODE == ROUND_SR_PHILOX) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      unsigned r = philox_word0(row_in_chunk * (unsigned)D + col + i, seed, 0u) & 0xFFFFFu;
+      t[i] = __uint_as_float((__float_as_uint(t[i]) + r) & 0xFFF00000u);
+    }
+  }
+  int packed = 0;
+  if (MODE == ROUND_SR_FAST) {
+    unsigned h = fast_mix(grow * (unsigned)(D / 4) + (col >> 2), seed);
+    packed = __builtin_amdgcn_cvt_sr_fp8_f32(clamp448(t[0]), fast_word(h, 0), packed, 0);
+    packed = __builtin_amdgcn_cvt_sr_fp8_f32(clamp448(t[1]), fast_word(h, 1), packed, 1);
+    packed = __builtin_amdgcn_cvt_sr_fp8_f32(clamp448(t[2]), fast_word(h, 2), packed, 2);
+    packed = __builtin_amdgcn_cvt_sr_fp8_f32(clamp448(t[3]), fast_word(h, 3), packed, 3);
+  } else {
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(t[0]), clamp448(t[1]), packed, false);
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(t[2]), clamp448(t[3]), packed, true);
+  }
+  return (unsigned)packed;
+}
+
+}  // namespace xmc

@@ -1,0 +1,429 @@
+// Fused FP8 extreme-classifier training step for gfx950 (MI355X).
+//
+// One persistent launch covers every label chunk of the layer.  Work unit = a tile of 64 consecutive
+// label rows of one chunk (64 x 768 e4m3 bytes, contiguous in HBM).  Two workgroups on the same XCD
+// form a pair and walk the same tile sequence: each brings the whole tile into LDS (the second read
+// is served by that XCD's L2), both compute the full logits tile, and each owns one half of the 768
+// input features for grad_X, grad_W and the in-place update, so every weight byte is read from HBM
+// once and written once per step and neither logits nor gradients ever reach memory.
+//
+// Per tile (4 wavefronts, wavefront w owns batch rows 32w..32w+31 for the logits and features
+// 96w..96w+95 of the workgroup's half for everything else):
+//   1. logits  Z[l,b]  = sum_k W[l,k] Xq[b,k]        v_mfma_f32_16x16x128_f8f6f4, Xq operands in registers
+//   2. G = bf16(sigmoid(bf16(Z)))  (-1 at positives)  written to LDS in [b][l] and [l][b] order
+//   3. grad_X[b,k] += sum_l G[l,b] W[l,k]             v_mfma_f32_16x16x32_bf16, W read with
+//                                                    ds_read_b64_tr_b8 (transposing LDS load), accumulators
+//                                                    stay in registers for the whole launch
+//   4. A[l,k]  = sum_b G[l,b] X[b,k]                 v_mfma_f32_16x16x32_bf16 (computed transposed)
+//   5. W[l,k]  = round(W[l,k] - lr * A[l,k])          in LDS, then 16-byte stores of whole rows
+// The next tile streams HBM -> LDS (global_load_lds, no registers) while the current one is processed.
+// The update is in place, so a workgroup may only write its half of a tile back once its partner holds
+// that tile in LDS: each workgroup publishes a tiles-loaded counter and checks its partner's before the
+// write-back (normally already satisfied; the wait is bounded and raises an error word instead of hanging).
+//
+// Reference semantics: src/xmc_classifiers/chunked_fp8xmc_clf.py:81-123 with
+// src/triton_kernels/matmul_kernel.py:204-239 (grad_X) and src/triton_kernels/fuse_kernel.py:63-113 (update).
+#include "xmc_common.h"
+
+namespace xmc {
+
+struct StepParams {
+  unsigned char* chunk[MAX_CHUNKS];   // device pointers of the chunk weight tensors [rows_per_chunk, 768] e4m3
+  unsigned seed[MAX_CHUNKS];          // per-chunk rounding seed
+  int num_chunks;
+  int rows_per_chunk;
+  int tiles_per_chunk;
+  int num_tiles;
+  const unsigned char* xq;            // logits operands (prep kernel layout)
+  const bf16x8* xt;                   // grad_W operands (prep kernel layout)
+  const unsigned* keys;               // sorted positives: label*256 + batch_row
+  const int* tile_ptr;                // [num_tiles+1] offsets into keys
+  floatx4* partial;                   // [gridDim.x][48][256] per-workgroup grad_X partial sums
+  int* flags;                         // [npairs][2] tiles-loaded counters of the two workgroups of a pair; [npairs*2] = error word
+  float zscale;                       // scale_w * scale_x applied to the logits accumulator
+  float lr_eff;                       // lr / scale_w
+  int batch;                          // real batch rows (<= BP)
+};
+
+typedef __attribute__((address_space(3))) unsigned char lds_u8;
+constexpr int SPIN_LIMIT = 1 << 20;   // polls of the partner's counter before giving up (error word set)
+
+// 32 bytes from a 16-byte aligned LDS address
+__device__ __forceinline__ intx8 lds_read32(const unsigned char* q) {
+  intx4 lo = *(const intx4*)q, hi = *(const intx4*)(q + 16);
+  return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+__device__ __forceinline__ void issue_tile_load(const unsigned char* gtile, int rows_valid, lds_u8* dst, int tid) {
+  // LDS image = 64 rows x 49 chunks of 16 bytes (48 data + 1 pad); wave-instruction j fills chunks
+  // [64j, 64j+63]; the pad chunk and rows past the end of the chunk re-read a valid address.
+  const int last_row = rows_valid - 1;
+#pragma unroll
+  for (int s = 0; s < 13; s++) {
+    int p = s * NT + tid;
+    if (p < TL * 49) {
+      int row = p / 49, c = p - row * 49;
+      row = row < last_row ? row : last_row;
+      c = c < 47 ? c : 47;
+      const unsigned char* g = gtile + (size_t)row * D + c * 16;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                       (__attribute__((address_space(3))) void*)(dst + (s * NT + (tid & ~63)) * 16), 16, 0, 0);
+    }
+  }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  unsigned char* wt0 = lds_raw;
+  unsigned char* gt = lds_raw + 2 * WT_BYTES;
+  unsigned char* gl = gt + BP * GT_S;
+
+  const int tid = threadIdx.x;
+  const int w = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int g = blockIdx.x;
+  const int xcd = g & 7, j = g >> 3, h = j & 1;
+  const int npairs = gridDim.x >> 1;
+  const int pair = (j >> 1) * 8 + xcd;
+  const int cw0 = HALF * h + WCOLS * w;          // first feature owned by this wavefront
+  const int cb0 = cw0 / 16;
+
+  // logits operands of this wavefront's 32 batch rows (re-read from L2 every tile: the register file is
+  // taken by the grad_X accumulators)
+  const intx8* xqw = (const intx8*)p.xq + (size_t)(w * 12) * 64 + lane;
+
+  floatx4 acc2[8][6];
+#pragma unroll
+  for (int a = 0; a < 8; a++)
+#pragma unroll
+    for (int b = 0; b < 6; b++) acc2[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  int t = pair;
+  if (t < p.num_tiles) {
+    int c = t / p.tiles_per_chunk, tj = t - c * p.tiles_per_chunk;
+    int row0 = tj * TL;
+    int rv = min(TL, p.rows_per_chunk - row0);
+    issue_tile_load(p.chunk[c] + (size_t)row0 * D, rv, (lds_u8*)wt0, tid);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  int* flag_mine = p.flags + 2 * pair + h;
+  int* flag_other = p.flags + 2 * pair + (h ^ 1);
+  if (tid == 0) __hip_atomic_store(flag_mine, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  for (int it = 0; t < p.num_tiles; t += npairs, it++) {
+    unsigned char* wt = wt0 + (it & 1) * WT_BYTES;
+    unsigned char* wtn = wt0 + ((it & 1) ^ 1) * WT_BYTES;
+    const int c = t / p.tiles_per_chunk, tj = t - c * p.tiles_per_chunk;
+    const int row0 = tj * TL;
+    const int rows_valid = min(TL, p.rows_per_chunk - row0);
+    unsigned char* gchunk = p.chunk[c];
+    const unsigned seed = p.seed[c];
+    const int p0 = p.tile_ptr[t], p1 = p.tile_ptr[t + 1];
+
+    // ---- 1. logits: Z[64 x 32] for batch rows 32w..32w+31
+    floatx4 z[4][2];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) { z[rb][0] = floatx4{0.f, 0.f, 0.f, 0.f}; z[rb][1] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++) {
+      const intx8 xq0 = xqw[(size_t)ks * 64], xq1 = xqw[(size_t)(6 + ks) * 64];
+#pragma unroll
+      for (int rb = 0; rb < 4; rb++) {
+        intx8 a = lds_read32(wt + (16 * rb + l16) * WS + ks * 128 + kg * 32);
+        z[rb][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq0, z[rb][0], 0, 0, 0, 0, 0, 0);
+        z[rb][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq1, z[rb][1], 0, 0, 0, 0, 0, 0);
+      }
+    }
+
+    // ---- 2. G = bf16(sigmoid(bf16(Z))), zero for rows past the end of the chunk
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+        const int b = 32 * w + 16 * nb + l16;
+        const int r0 = 16 * rb + 4 * kg;
+        unsigned short s[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float zf = bf16_rt(z[rb][nb][i] * p.zscale);
+          float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-zf));
+          s[i] = (r0 + i < rows_valid) ? bf16_bits(sg) : (unsigned short)0;
+          *(unsigned short*)(gl + (r0 + i) * GL_S + b * 2) = s[i];
+        }
+        uint2 v;
+        v.x = (unsigned)s[0] | ((unsigned)s[1] << 16);
+        v.y = (unsigned)s[2] | ((unsigned)s[3] << 16);
+        *(uint2*)(gt + b * GT_S + r0 * 2) = v;
+      }
+    }
+    __syncthreads();
+
+    // ---- stream the next tile into the other LDS buffer (every wavefront has finished reading it:
+    //      its last readers were the write-back loads of the previous iteration)
+    const int tn = t + npairs;
+    if (tn < p.num_tiles) {
+      int cn = tn / p.tiles_per_chunk, tjn = tn - cn * p.tiles_per_chunk;
+      int row0n = tjn * TL;
+      issue_tile_load(p.chunk[cn] + (size_t)row0n * D, min(TL, p.rows_per_chunk - row0n), (lds_u8*)wtn, tid);
+    }
+    int seen = __hip_atomic_load(flag_other, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // ---- positives of this tile: G -= 1 (set semantics: a repeated key is applied once)
+    if (p1 > p0) {
+      const unsigned label0 = (unsigned)(c * p.rows_per_chunk + row0);
+      for (int e = p0 + tid; e < p1; e += NT) {
+        unsigned key = p.keys[e];
+        if (e > 0 && p.keys[e - 1] == key) continue;
+        unsigned b = key & 255u, l = (key >> 8) - label0;
+        if (b < (unsigned)BP && l < (unsigned)rows_valid) {
+          unsigned short* q = (unsigned short*)(gl + l * GL_S + b * 2);
+          unsigned short s2 = bf16_bits(bf16_from_bits(*q) - 1.0f);
+          *q = s2;
+          *(unsigned short*)(gt + b * GT_S + l * 2) = s2;
+        }
+      }
+      __syncthreads();
+    }
+
+    // ---- 3. grad_X[128 x 96 of this wavefront] += G^T W
+#pragma unroll 1
+    for (int ks2 = 0; ks2 < 2; ks2++) {
+      bf16x8 ga[8];
+#pragma unroll
+      for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gt + (16 * mb + l16) * GT_S + ks2 * 64 + kg * 16);
+#pragma unroll
+      for (int nn = 0; nn < 6; nn++) {
+        const unsigned char* src = wt + (32 * ks2 + 8 * kg + (l16 >> 1)) * WS + cw0 + 16 * nn + (l16 & 1) * 8;
+        intx2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(lds_u8*)src);
+        floatx2 f01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, false), f23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, true);
+        floatx2 f45 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, false), f67 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, true);
+        bf16x8 wb = {(__bf16)f01.x, (__bf16)f01.y, (__bf16)f23.x, (__bf16)f23.y,
+                     (__bf16)f45.x, (__bf16)f45.y, (__bf16)f67.x, (__bf16)f67.y};
+#pragma unroll
+        for (int mb = 0; mb < 8; mb++)
+          acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb, acc2[mb][nn], 0, 0, 0);
+      }
+    }
+
+    // ---- 4+5. A^T[96 x 64] = X^T G^T, then the update of this wavefront's 96 features, in LDS
+#pragma unroll 1
+    for (int half = 0; half < 2; half++) {
+      floatx4 acc3[3][4];
+#pragma unroll
+      for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc3[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) {
+        bf16x8 bg[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) bg[nb] = *(const bf16x8*)(gl + (16 * nb + l16) * GL_S + ks * 64 + kg * 16);
+#pragma unroll
+        for (int m3 = 0; m3 < 3; m3++) {
+          bf16x8 ax = p.xt[(size_t)((cb0 + half * 3 + m3) * 4 + ks) * 64 + lane];
+#pragma unroll
+          for (int nb = 0; nb < 4; nb++)
+            acc3[m3][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bg[nb], acc3[m3][nb], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int m3 = 0; m3 < 3; m3++) {
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+          const int row = 16 * nb + l16;
+          const int col = cw0 + 16 * (half * 3 + m3) + 4 * kg;
+          unsigned* wp = (unsigned*)(wt + row * WS + col);
+          unsigned wq = *wp;
+          floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq, true);
+          floatx4 a = acc3[m3][nb];
+          float t0 = __builtin_fmaf(-p.lr_eff, a[0], w01.x), t1 = __builtin_fmaf(-p.lr_eff, a[1], w01.y);
+          float t2 = __builtin_fmaf(-p.lr_eff, a[2], w23.x), t3 = __builtin_fmaf(-p.lr_eff, a[3], w23.y);
+          *wp = round4<MODE>(t0, t1, t2, t3, (unsigned)(row0 + row), (unsigned)(c * p.rows_per_chunk + row0 + row),
+                             (unsigned)col, seed);
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // next tile has landed in LDS (this thread's part)
+    __syncthreads();
+    if (tid == 0) __hip_atomic_store(flag_mine, it + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the partner must hold this tile before its rows are overwritten
+    for (int spin = 0; seen < it + 1; spin++) {
+      if (spin >= SPIN_LIMIT) { p.flags[2 * npairs] = 1; break; }
+      __builtin_amdgcn_s_sleep(2);
+      seen = __hip_atomic_load(flag_other, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- write this workgroup's half of the updated tile back, 16 bytes per lane, whole 128-byte lines
+#pragma unroll
+    for (int s = 0; s < 6; s++) {
+      int ch = s * NT + tid;
+      int row = ch / 24, cc = ch - row * 24;
+      if (row < rows_valid) {
+        uint4 v = *(const uint4*)(wt + row * WS + HALF * h + cc * 16);
+        *(uint4*)(gchunk + (size_t)(row0 + row) * D + HALF * h + cc * 16) = v;
+      }
+    }
+  }
+
+  // ---- per-workgroup grad_X partial, summed in a fixed order by reduce_gx_kernel
+  floatx4* dst = p.partial + (size_t)g * 48 * NT;
+#pragma unroll
+  for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+    for (int nn = 0; nn < 6; nn++) dst[(mb * 6 + nn) * NT + tid] = acc2[mb][nn];
+}
+
+// grad_X = scale * sum over workgroups of the partials; writes fp32 and bf16 [batch, 768]
+__global__ void reduce_gx_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32, unsigned short* gx_bf16,
+                                 int batch) {
+  const int slot = blockIdx.x >> 1, h = blockIdx.x & 1;   // slot = mb*6+nn
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int g = 0; g < nwg; g++) {
+    if (((g >> 3) & 1) != h) continue;
+    floatx4 v = partial[((size_t)g * 48 + slot) * NT + tid];
+    s += v;
+  }
+  const int mb = slot / 6, nn = slot - mb * 6;
+  const int col = HALF * h + WCOLS * w + 16 * nn + l16;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int b = 16 * mb + 4 * kg + i;
+    if (b < batch) {
+      float v = s[i] * scale;
+      if (gx_f32) gx_f32[(size_t)b * D + col] = v;
+      if (gx_bf16) gx_bf16[(size_t)b * D + col] = bf16_bits(v);
+    }
+  }
+}
+
+// Build the operand images of X used by the step kernel.
+//   xq: e4m3(X / scale_x) in v_mfma 16x16x128 B-operand order: [(w*2+nb)*6+ks][lane][32 bytes]
+//   xt: bf16 X^T in v_mfma 16x16x32 A-operand order: [(col/16)*4+ks][lane][8 bf16], lane = (col%16) + 16*kg,
+//       element j = X[32ks + 8kg + j][col]
+__global__ void prep_x_kernel(const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq, unsigned short* xt) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (b, k4) group of 4 features
+  if (i >= BP * (D / 4)) return;
+  int b = i / (D / 4), k = (i - b * (D / 4)) * 4;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  unsigned short raw[4] = {0, 0, 0, 0};
+  if (b < batch) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) { raw[q] = x[(size_t)b * D + k + q]; v[q] = bf16_from_bits(raw[q]) * inv_scale_x; }
+  }
+  int packed = 0;
+  packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v[0]), clamp448(v[1]), packed, false);
+  packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v[2]), clamp448(v[3]), packed, true);
+  {
+    int w = b >> 5, nb = (b >> 4) & 1, n = b & 15;
+    int ks = k >> 7, kgq = (k >> 5) & 3, jq = k & 31;
+    size_t off = ((size_t)((w * 2 + nb) * 6 + ks) * 64 + (n + 16 * kgq)) * 32 + jq;
+    *(int*)(xq + off) = packed;
+  }
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    int col = k + q;
+    int ks = b >> 5, kgq = (b >> 3) & 3, jq = b & 7;
+    size_t off = ((size_t)((col >> 4) * 4 + ks) * 64 + ((col & 15) + 16 * kgq)) * 8 + jq;
+    xt[off] = raw[q];
+  }
+}
+
+// Sort the positives of one step and drop nothing: key = label*256 + batch_row, invalid entries -> 0xFFFFFFFF.
+// Single workgroup, bitonic network in LDS (n_pad = power of two <= MAX_POS).
+__global__ __launch_bounds__(1024) void sort_keys_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys) {
+  extern __shared__ unsigned sk[];
+  for (int i = threadIdx.x; i < n_pad; i += blockDim.x) {
+    unsigned key = 0xFFFFFFFFu;
+    if (i < nnz) {
+      int r = coo[2 * i], l = coo[2 * i + 1];
+      if (r >= 0 && r < batch && l >= 0 && l < (1 << 24) - 1) key = ((unsigned)l << 8) | (unsigned)r;
+    }
+    sk[i] = key;
+  }
+  __syncthreads();
+  for (int k = 2; k <= n_pad; k <<= 1) {
+    for (int jj = k >> 1; jj > 0; jj >>= 1) {
+      for (int i = threadIdx.x; i < n_pad; i += blockDim.x) {
+        int ixj = i ^ jj;
+        if (ixj > i) {
+          unsigned a = sk[i], b = sk[ixj];
+          bool up = (i & k) == 0;
+          if ((a > b) == up) { sk[i] = b; sk[ixj] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = threadIdx.x; i < n_pad; i += blockDim.x) keys[i] = sk[i];
+}
+
+// tile_ptr[t] = first key whose label >= first label of tile t; tile_ptr[num_tiles] = first key past the last tile
+__global__ void tile_ptr_kernel(const unsigned* keys, int n_pad, int rows_per_chunk, int tiles_per_chunk, int num_tiles,
+                                int* tile_ptr) {
+  int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t > num_tiles) return;
+  unsigned long long label0;
+  if (t == num_tiles) {
+    label0 = (unsigned long long)(num_tiles / tiles_per_chunk) * rows_per_chunk;
+  } else {
+    int c = t / tiles_per_chunk, tj = t - c * tiles_per_chunk;
+    label0 = (unsigned long long)c * rows_per_chunk + (unsigned long long)tj * TL;
+  }
+  unsigned long long bound = label0 << 8;
+  int lo = 0, hi = n_pad;
+  while (lo < hi) {
+    int mid = (lo + hi) >> 1;
+    if ((unsigned long long)keys[mid] < bound) lo = mid + 1; else hi = mid;
+  }
+  tile_ptr[t] = lo;
+}
+
+// Inference logits: out[b, label] = bf16(zscale * sum_k Xq[b,k] W[label,k]) for one chunk.
+__global__ __launch_bounds__(NT) void fp8_forward_kernel(const unsigned char* wchunk, int rows, const unsigned char* xqimg,
+                                                         float zscale, unsigned short* out, long long out_stride,
+                                                         long long label_base, long long num_labels, int batch) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  intx8 xq[2][6];
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++)
+      xq[nb][ks] = *(const intx8*)(xqimg + ((size_t)((w * 2 + nb) * 6 + ks) * 64 + lane) * 32);
+  const int ntiles = (rows + TL - 1) / TL;
+  for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int row0 = t * TL, rows_valid = min(TL, rows - row0);
+    __syncthreads();
+    issue_tile_load(wchunk + (size_t)row0 * D, rows_valid, (lds_u8*)lds_raw, tid);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    floatx4 z[4][2];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) { z[rb][0] = floatx4{0.f, 0.f, 0.f, 0.f}; z[rb][1] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++)
+#pragma unroll
+      for (int rb = 0; rb < 4; rb++) {
+        intx8 a = lds_read32(lds_raw + (16 * rb + l16) * WS + ks * 128 + kg * 32);
+        z[rb][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq[0][ks], z[rb][0], 0, 0, 0, 0, 0, 0);
+        z[rb][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq[1][ks], z[rb][1], 0, 0, 0, 0, 0, 0);
+      }
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++)
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++) {
+        const int b = 32 * w + 16 * nb + l16;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          int r = 16 * rb + 4 * kg + i;
+          long long label = label_base + row0 + r;
+          if (r < rows_valid && b < batch && label < num_labels)
+            out[(size_t)b * out_stride + label] = bf16_bits(z[rb][nb][i] * zscale);
+        }
+      }
+  }
+}
+
+}  // namespace xmc

@@ -1,0 +1,97 @@
+"""Tensor-level wrappers over the C ABI.  torch supplies device memory and the current stream only."""
+import ctypes
+
+import torch
+
+from . import _lib
+
+FEATURES = 768
+MAX_BATCH = 128
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _chunk_array(chunks):
+    arr = (ctypes.c_void_p * len(chunks))()
+    rows = chunks[0].shape[0]
+    for i, c in enumerate(chunks):
+        assert c.is_cuda and c.is_contiguous(), "weight chunks must be contiguous device tensors"
+        assert c.dtype in (torch.float8_e4m3fn, torch.uint8) and c.shape == (rows, FEATURES), \
+            "weight chunks must be equal-sized [rows, 768] e4m3fn tensors"
+        arr[i] = c.data_ptr()
+    return arr, rows
+
+
+def workspace_bytes(num_chunks, rows_per_chunk):
+    n = _lib.load().xmc_workspace_bytes(num_chunks, rows_per_chunk)
+    if n == 0:
+        raise _lib.XmcError("unsupported chunk geometry")
+    return n
+
+
+def alloc_workspace(num_chunks, rows_per_chunk, device):
+    return torch.empty(workspace_bytes(num_chunks, rows_per_chunk), dtype=torch.uint8, device=device)
+
+
+def fp8_step(chunks, x, labels, lr, seeds=None, round_mode="rtn", scale_w=1.0, scale_x=1.0, workspace=None,
+             grad_out=None, want_f32=False):
+    """One fused training step (reference: chunked_fp8xmc_clf.py:81-123).  Updates `chunks` in place and returns
+    grad_input (bf16 [B, 768]) or (grad_input, grad_x_fp32) when want_f32."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2
+    assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
+    assert labels.dim() == 2 and labels.shape[1] == 2
+    batch, feat = x.shape
+    arr, rows = _chunk_array(chunks)
+    nc = len(chunks)
+    if workspace is None:
+        workspace = alloc_workspace(nc, rows, x.device)
+    if grad_out is None:
+        grad_out = torch.empty(batch, feat, dtype=torch.bfloat16, device=x.device)
+    gf = torch.empty(batch, feat, dtype=torch.float32, device=x.device) if want_f32 else None
+    sarr = None
+    if seeds is not None:
+        sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
+    st = lib.xmc_fp8_step(arr, nc, rows, x.data_ptr(), batch, feat, labels.data_ptr() if labels.numel() else None,
+                          labels.shape[0], float(lr), sarr, _lib.ROUND_MODES[round_mode], float(scale_w),
+                          float(scale_x), grad_out.data_ptr(), gf.data_ptr() if gf is not None else None,
+                          workspace.data_ptr(), workspace.numel(), _stream_ptr())
+    _lib.check(st, "xmc_fp8_step")
+    return (grad_out, gf) if want_f32 else grad_out
+
+
+def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None):
+    """Inference logits [B, num_labels] bf16 (reference: chunked_fp8xmc_clf.py:45-60).  Any batch size: rows are
+    processed in slices of at most 128, the last one padded to a multiple of 16."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dim() == 2 and x.shape[1] == FEATURES
+    xb = x.to(torch.bfloat16).contiguous()      # exact for e4m3 input
+    arr, rows = _chunk_array(chunks)
+    nc = len(chunks)
+    if workspace is None:
+        workspace = alloc_workspace(nc, rows, x.device)
+    total = xb.shape[0]
+    out = torch.empty(total, num_labels, dtype=torch.bfloat16, device=x.device)
+    for lo in range(0, total, MAX_BATCH):
+        hi = min(lo + MAX_BATCH, total)
+        n = hi - lo
+        npad = (n + 15) // 16 * 16
+        xs = xb[lo:hi]
+        if npad != n:
+            xs = torch.cat([xs, torch.zeros(npad - n, FEATURES, dtype=xb.dtype, device=xb.device)])
+            tmp = torch.empty(npad, num_labels, dtype=torch.bfloat16, device=x.device)
+        else:
+            tmp = out[lo:hi]
+        st = lib.xmc_fp8_forward(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
+                                 tmp.data_ptr(), num_labels, num_labels, workspace.data_ptr(), workspace.numel(),
+                                 _stream_ptr())
+        _lib.check(st, "xmc_fp8_forward")
+        if npad != n:
+            out[lo:hi] = tmp[:n]
+    return out
+
+
+def step_error_word(workspace, num_chunks, rows_per_chunk):
+    return _lib.load().xmc_step_error_word(workspace.data_ptr(), num_chunks, rows_per_chunk, _stream_ptr())

@@ -1,0 +1,84 @@
+/* C ABI of the MI355X (gfx950) extreme-classifier step library, libelmo_xmc.so.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream (passed as void*), enqueues its
+ * kernels on that stream and returns immediately with a status code (0 = ok, negative = error, see
+ * xmc_error_string).  Nothing here allocates or frees device memory, synchronises the device or copies
+ * to the host: the caller owns every buffer, including the workspace.
+ *
+ * The entry points replace, for the FP8 layer of the reference
+ *   src/xmc_classifiers/chunked_fp8xmc_clf.py:81-123   Fp8XMCBCEChunkedLayer.xfc_forward_backward
+ *   src/xmc_classifiers/chunked_fp8xmc_clf.py:45-60    Fp8XMCBCEChunkedLayer.xfc_forward
+ * and the kernels those call
+ *   torch._scaled_mm (:101-102), sigmoid_/index_put (:107-108),
+ *   src/triton_kernels/matmul_kernel.py:342-353 large_k_matmul,
+ *   src/triton_kernels/fuse_kernel.py:116-131 matmul_update.
+ */
+#ifndef ELMO_XMC_H
+#define ELMO_XMC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  XMC_OK = 0,
+  XMC_ERR_NULL = -1,        /* a required pointer is null */
+  XMC_ERR_SHAPE = -2,       /* unsupported shape (features != 768, batch > 128 or not a multiple of 16, rows % 16 != 0, ...) */
+  XMC_ERR_ALIGN = -3,       /* a device pointer is not 16-byte aligned */
+  XMC_ERR_RANGE = -4,       /* too many chunks / positives / labels for this build */
+  XMC_ERR_WORKSPACE = -5,   /* workspace smaller than xmc_workspace_bytes() */
+  XMC_ERR_MODE = -6,        /* unknown rounding mode */
+  XMC_ERR_LAUNCH = -7,      /* HIP reported a launch failure */
+  XMC_ERR_DEVICE = -8       /* not a gfx950 device / too few compute units */
+};
+
+/* rounding of the updated weights (fuse_kernel.py:107-113 is XMC_ROUND_SR_PHILOX) */
+enum {
+  XMC_ROUND_RTN = 0,        /* round to nearest even, saturating at +-448 */
+  XMC_ROUND_SR_PHILOX = 1,  /* the reference bit recipe: Philox-4x32-10 word per element, add 20 bits, mask, cast */
+  XMC_ROUND_SR_FAST = 2     /* unbiased stochastic rounding on the e4m3 grid (hardware converter, counter hash) */
+};
+
+int xmc_version(void);
+const char* xmc_error_string(int status);
+
+/* Bytes of workspace the step needs for `num_chunks` chunks of `rows_per_chunk` rows (features fixed at 768).
+ * Returns 0 for an unsupported shape. */
+size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk);
+
+/* One training step over all chunks: logits, sigmoid minus sparse targets, grad_X, grad_W and the in-place
+ * SGD update (chunked_fp8xmc_clf.py:91-123).
+ *   chunk_ptrs      host array of num_chunks device pointers, each [rows_per_chunk, 768] e4m3fn, updated in place
+ *   x_bf16          device [batch, 768] bf16 (not modified); batch % 16 == 0, batch <= 128
+ *   labels_coo      device [nnz, 2] int32 (row-in-batch, label id in the padded label space), any order, duplicates allowed
+ *   lr              learning rate (xmc_lr[0])
+ *   seeds           host array of num_chunks seeds (one torch.randint(0, 1e6) per chunk in the reference, :113)
+ *   round_mode      XMC_ROUND_*
+ *   scale_w/scale_x per-tensor scales: weight = scale_w * code, Xq = e4m3(X / scale_x); the reference uses 1, 1
+ *   grad_x_bf16     device [batch, 768] bf16 out (self.grad_input, :122)
+ *   grad_x_f32      device [batch, 768] fp32 out, or null
+ */
+int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                 int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                 float scale_w, float scale_x, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
+/* Inference logits (chunked_fp8xmc_clf.py:45-60): out[b, label] = bf16(scale * sum_k e4m3(X/scale_x)[b,k] * W[label,k])
+ * for label < num_labels (the padding rows of the last chunk are dropped, :60).
+ *   out_bf16        device [batch, out_stride] bf16, out_stride >= num_labels
+ */
+int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                    int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
+                    long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Reads back the error word a step leaves in the workspace (non-zero: a workgroup gave up waiting for its
+ * partner).  Synchronises the stream; meant for tests and debugging, not for the training loop. */
+int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
