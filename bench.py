@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused extreme-classifier training step on one MI355X.
+
+One "step" = one call of the FP8 layer's xfc_forward_backward over all label chunks (the hot path of
+src/xmc_classifiers/chunked_fp8xmc_clf.py:81-123): X[128,768] bf16 resident in HBM, W[670091(+pad),768] e4m3
+resident in HBM, positives as COO int32.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2_fp8_670k] [--round sr_fast|sr_philox|rtn]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP8_PEAK_TFLOPS = 5000.0
+
+
+def padded_labels(num_labels, num_chunks):
+    # src/xmc_classifiers/chunked_fp8xmc_clf.py:26
+    return num_labels + 16 * num_chunks - num_labels % (16 * num_chunks)
+
+
+def cpu_baseline(cfg, budget_s=20.0):
+    """The reference's PyTorch CPU bf16 chunked path (oracle.torch_port) on ONE chunk of this workload,
+    scaled by the number of chunks."""
+    import numpy as np
+    import torch
+    from elmo_amd import synth
+    from oracle import torch_port
+    nc = cfg.num_chunks
+    rows = padded_labels(cfg.num_labels, nc) // nc
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(cfg.seed)
+    w = (torch.randn(rows, cfg.dim, generator=g) * cfg.init_std).to(torch.bfloat16)
+    x = torch.from_numpy(synth.make_x(cfg.batch, cfg.dim, cfg.seed)).to(torch.bfloat16)
+    lab = synth.make_labels(cfg.batch, cfg.num_labels, cfg.pos_mean, cfg.zipf_s, cfg.seed)
+    lab = torch.from_numpy(lab[lab[:, 1] < rows])
+    torch_port.bf16_chunked_step(w, x, lab, cfg.lr, 1)          # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start < budget_s or len(times) < 2):
+        t0 = time.perf_counter()
+        torch_port.bf16_chunked_step(w, x, lab, cfg.lr, 1)
+        times.append(time.perf_counter() - t0)
+    t_chunk = float(np.median(times))
+    return {
+        "value": 1.0 / (t_chunk * nc), "unit": "steps/s", "cores": threads, "kind": "port",
+        "sample": f"1 of {nc} chunks ({rows} labels x {cfg.dim}, batch {cfg.batch}), bf16 weights, round-to-nearest "
+                  f"update, median of {len(times)} runs, step time scaled by {nc}",
+        "seconds_per_chunk": t_chunk,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="cfg2_fp8_670k")
+    ap.add_argument("--round", default="sr_fast", choices=["sr_fast", "sr_philox", "rtn"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the classifier step on ONE GPU; --gpus > 1 is not supported "
+              "(the path shards by label rows, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from elmo_amd import _lib, ops, synth
+
+    cfg = synth.CONFIGS[args.config]
+    if cfg.batch > ops.MAX_BATCH or cfg.weights != "e4m3":
+        print(f"bench.py: config {cfg.name} is not runnable by this build yet", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+    nc = cfg.num_chunks
+    L_pad = padded_labels(cfg.num_labels, nc)
+    rows = L_pad // nc
+
+    # ---- resident inputs (synthetic, seeded)
+    gen = torch.Generator(device=dev).manual_seed(cfg.seed)
+    chunks = []
+    for _ in range(nc):
+        w = torch.randn(rows, cfg.dim, generator=gen, device=dev, dtype=torch.float32) * cfg.init_std
+        chunks.append(w.to(torch.float8_e4m3fn))
+        del w
+    x_np = synth.make_x(cfg.batch, cfg.dim, cfg.seed)
+    x = torch.from_numpy(x_np).to(dev).to(torch.bfloat16)
+    labels = torch.from_numpy(synth.make_labels(cfg.batch, cfg.num_labels, cfg.pos_mean, cfg.zipf_s, cfg.seed)).to(dev)
+    torch.cuda.synchronize()
+    weight_bytes = sum(c.numel() for c in chunks)
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    base_alloc = torch.cuda.memory_allocated()
+
+    workspace = ops.alloc_workspace(nc, rows, dev)
+    grad = torch.empty(cfg.batch, cfg.dim, dtype=torch.bfloat16, device=dev)
+    seed_rng = np.random.default_rng(cfg.seed)
+
+    def one_step():
+        seeds = seed_rng.integers(0, 1_000_000, size=nc)
+        ops.fp8_step(chunks, x, labels, cfg.lr, seeds=seeds, round_mode=args.round, workspace=workspace, grad_out=grad)
+
+    # HIP events around the fused kernel of every timed step, on the stream the kernel is launched on
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    events = []
+    for _ in range(args.steps):
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
+        events.append((a, b))
+
+    for _ in range(args.warmup):
+        one_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        lib.xmc_profile_events(events[i][0], events[i][1])
+        one_step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    err = ops.step_error_word(workspace, nc, rows)
+    assert err == 0, "a workgroup timed out waiting for its partner"
+    assert bool(torch.isfinite(grad.float()).all())
+
+    kms = []
+    for a, b in events:
+        ms = ctypes.c_float()
+        assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+        kms.append(ms.value)
+    kernel_ms = float(np.mean(kms))
+    ms_per_step = elapsed / args.steps * 1e3
+    steps_per_s = args.steps / elapsed
+    peak_bytes = torch.cuda.max_memory_allocated() - base_alloc + weight_bytes
+
+    algo_bytes = 2.0 * cfg.num_labels * cfg.dim * 1          # each weight byte read once, written once
+    algo_flops = 6.0 * cfg.batch * cfg.num_labels * cfg.dim
+    t_roof = max(algo_flops / (FP8_PEAK_TFLOPS * 1e12), algo_bytes / (HBM_PEAK_GBS * 1e9))
+    achieved_gbs = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"{cfg.name}:{args.round}")
+
+    out = {
+        "metric": "XMC classifier train steps/sec at 670K labels FP8",
+        "value": steps_per_s, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 weights+logits MFMA, bf16 gradient MFMA, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": cfg.name, "labels": cfg.num_labels, "labels_padded": L_pad, "features": cfg.dim,
+                   "batch": cfg.batch, "chunks": nc, "rows_per_chunk": rows, "positives": int(labels.shape[0]),
+                   "lr": cfg.lr, "rounding": args.round, "seed": cfg.seed},
+        "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "fp8_step_kernel", "kernel_ms": kernel_ms,
+                     "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_flops_per_launch": algo_flops},
+        "roofline_step_frac": t_roof / (ms_per_step * 1e-3),
+        "roofline_steps_per_s": 1.0 / t_roof,
+        "peak_hbm_gb": peak_bytes / 1e9, "peak_hbm_over_weights": peak_bytes / weight_bytes,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

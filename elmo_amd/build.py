@@ -1,0 +1,27 @@
+"""Compiles the HIP sources of this package for gfx950 into elmo_amd/libelmo_xmc.so (in-tree)."""
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "csrc", "xmc_capi.hip")
+OUT = os.path.join(HERE, "libelmo_xmc.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-munsafe-fp-atomics",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def build(verbose=False):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + HIPCC_FLAGS + [SRC, "-o", OUT]
+    if verbose:
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+    return res.stderr if verbose else OUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

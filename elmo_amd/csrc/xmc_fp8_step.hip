@@ -45,8 +45,27 @@ struct StepParams {
   int batch;                          // real batch rows (<= BP)
 };
 
+#ifndef XMC_DBG_SKIP
+#define XMC_DBG_SKIP 0   // timing experiments only: bit mask of phases to leave out (results are then wrong)
+#endif
 typedef __attribute__((address_space(3))) unsigned char lds_u8;
 constexpr int SPIN_LIMIT = 1 << 20;   // polls of the partner's counter before giving up (error word set)
+
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point
+
+// eight e4m3 codes -> eight bf16 values (exact)
+__device__ __forceinline__ bf16x8 fp8x8_to_bf16x8(intx2 raw) {
+  floatx2 f01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, false), f23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, true);
+  floatx2 f45 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, false), f67 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, true);
+  return bf16x8{(__bf16)f01.x, (__bf16)f01.y, (__bf16)f23.x, (__bf16)f23.y,
+                (__bf16)f45.x, (__bf16)f45.y, (__bf16)f67.x, (__bf16)f67.y};
+}
+
+// transposing LDS read: within each group of 16 lanes, lanes 2j and 2j+1 point at the two 8-byte halves of
+// a 16-byte row j (j = 0..7); lane i receives byte i of rows 0..7
+__device__ __forceinline__ intx2 lds_tr8(const unsigned char* q) {
+  return __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(__attribute__((address_space(3))) unsigned char*)q);
+}
 
 // 32 bytes from a 16-byte aligned LDS address
 __device__ __forceinline__ intx8 lds_read32(const unsigned char* q) {
@@ -91,6 +110,11 @@ __global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
   // logits operands of this wavefront's 32 batch rows (re-read from L2 every tile: the register file is
   // taken by the grad_X accumulators)
   const intx8* xqw = (const intx8*)p.xq + (size_t)(w * 12) * 64 + lane;
+  // ring of three K steps of logits operands (two 16-row batch blocks each); steps 0 and 1 are requested
+  // before the tile loop and again at the end of every iteration, step ks+2 while step ks is consumed
+  intx8 xqb[3][2];
+  xqb[0][0] = xqw[0]; xqb[0][1] = xqw[6 * 64];
+  xqb[1][0] = xqw[1 * 64]; xqb[1][1] = xqw[7 * 64];
 
   floatx4 acc2[8][6];
 #pragma unroll
@@ -121,40 +145,58 @@ __global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
     const unsigned seed = p.seed[c];
     const int p0 = p.tile_ptr[t], p1 = p.tile_ptr[t + 1];
 
-    // ---- 1. logits: Z[64 x 32] for batch rows 32w..32w+31
+    // ---- 1. logits: Z[64 x 32] for batch rows 32w..32w+31; 24 steps (ks major, row block minor), the LDS
+    //         operand of step s+2 is requested before the two MFMAs of step s are issued
     floatx4 z[4][2];
 #pragma unroll
     for (int rb = 0; rb < 4; rb++) { z[rb][0] = floatx4{0.f, 0.f, 0.f, 0.f}; z[rb][1] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+    if (!(XMC_DBG_SKIP & 1)) {
+      const unsigned char* abase = wt + l16 * WS + kg * 32;
+      intx8 ab[3];
+      ab[0] = lds_read32(abase);
+      ab[1] = lds_read32(abase + 16 * WS);
 #pragma unroll
-    for (int ks = 0; ks < 6; ks++) {
-      const intx8 xq0 = xqw[(size_t)ks * 64], xq1 = xqw[(size_t)(6 + ks) * 64];
-#pragma unroll
-      for (int rb = 0; rb < 4; rb++) {
-        intx8 a = lds_read32(wt + (16 * rb + l16) * WS + ks * 128 + kg * 32);
-        z[rb][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq0, z[rb][0], 0, 0, 0, 0, 0, 0);
-        z[rb][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq1, z[rb][1], 0, 0, 0, 0, 0, 0);
+      for (int s = 0; s < 24; s++) {
+        const int ks = s >> 2, rb = s & 3;
+        if (s + 2 < 24) ab[(s + 2) % 3] = lds_read32(abase + 16 * ((s + 2) & 3) * WS + ((s + 2) >> 2) * 128);
+        if (rb == 0 && ks + 2 < 6) {
+          xqb[(ks + 2) % 3][0] = xqw[(size_t)(ks + 2) * 64];
+          xqb[(ks + 2) % 3][1] = xqw[(size_t)(6 + ks + 2) * 64];
+        }
+        SCHED_FENCE();
+        z[rb][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ab[s % 3], xqb[ks % 3][0], z[rb][0], 0, 0, 0, 0, 0, 0);
+        z[rb][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ab[s % 3], xqb[ks % 3][1], z[rb][1], 0, 0, 0, 0, 0, 0);
+        SCHED_FENCE();
       }
     }
 
     // ---- 2. G = bf16(sigmoid(bf16(Z))), zero for rows past the end of the chunk
+    {
+      const float nlog2e = -1.44269504088896340736f;
 #pragma unroll
-    for (int rb = 0; rb < 4; rb++) {
+      for (int rb = 0; rb < 4; rb++) {
 #pragma unroll
-      for (int nb = 0; nb < 2; nb++) {
-        const int b = 32 * w + 16 * nb + l16;
-        const int r0 = 16 * rb + 4 * kg;
-        unsigned short s[4];
+        for (int nb = 0; nb < 2; nb++) {
+          const int b = 32 * w + 16 * nb + l16;
+          const int r0 = 16 * rb + 4 * kg;
+          unsigned short sb[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          float zf = bf16_rt(z[rb][nb][i] * p.zscale);
-          float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-zf));
-          s[i] = (r0 + i < rows_valid) ? bf16_bits(sg) : (unsigned short)0;
-          *(unsigned short*)(gl + (r0 + i) * GL_S + b * 2) = s[i];
+          for (int i = 0; i < 4; i++) {
+            float zf = bf16_rt(z[rb][nb][i] * p.zscale);
+            float sg = (XMC_DBG_SKIP & 2) ? zf : __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * nlog2e));
+            sb[i] = bf16_bits(sg);
+          }
+          if (rows_valid < TL) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) sb[i] = (r0 + i < rows_valid) ? sb[i] : (unsigned short)0;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; i++) *(unsigned short*)(gl + (r0 + i) * GL_S + b * 2) = sb[i];
+          uint2 v;
+          v.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
+          v.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
+          *(uint2*)(gt + b * GT_S + r0 * 2) = v;
         }
-        uint2 v;
-        v.x = (unsigned)s[0] | ((unsigned)s[1] << 16);
-        v.y = (unsigned)s[2] | ((unsigned)s[3] << 16);
-        *(uint2*)(gt + b * GT_S + r0 * 2) = v;
       }
     }
     __syncthreads();
@@ -162,7 +204,7 @@ __global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
     // ---- stream the next tile into the other LDS buffer (every wavefront has finished reading it:
     //      its last readers were the write-back loads of the previous iteration)
     const int tn = t + npairs;
-    if (tn < p.num_tiles) {
+    if (tn < p.num_tiles && !(XMC_DBG_SKIP & 32)) {
       int cn = tn / p.tiles_per_chunk, tjn = tn - cn * p.tiles_per_chunk;
       int row0n = tjn * TL;
       issue_tile_load(p.chunk[cn] + (size_t)row0n * D, min(TL, p.rows_per_chunk - row0n), (lds_u8*)wtn, tid);
@@ -186,69 +228,100 @@ __global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
       __syncthreads();
     }
 
-    // ---- 3. grad_X[128 x 96 of this wavefront] += G^T W
-#pragma unroll 1
-    for (int ks2 = 0; ks2 < 2; ks2++) {
-      bf16x8 ga[8];
+    // ---- 3. grad_X[128 x 96 of this wavefront] += G^T W; 12 steps (32-row K step major, 16-feature block
+    //         minor); the transposed W read of step s+2 and the fp8->bf16 conversion of step s+1 are
+    //         issued between the MFMAs of step s
+    if (!(XMC_DBG_SKIP & 4)) {
+      const unsigned char* wsrc = wt + (8 * kg + (l16 >> 1)) * WS + cw0 + (l16 & 1) * 8;
+      const unsigned char* gsrc = gt + l16 * GT_S + kg * 16;
+      bf16x8 ga[2][8];
 #pragma unroll
-      for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gt + (16 * mb + l16) * GT_S + ks2 * 64 + kg * 16);
+      for (int mb = 0; mb < 8; mb++) ga[0][mb] = *(const bf16x8*)(gsrc + 16 * mb * GT_S);
+      intx2 raw[3];
+      raw[0] = lds_tr8(wsrc);
+      raw[1] = lds_tr8(wsrc + 16);
+      bf16x8 wb[2];
+      wb[0] = fp8x8_to_bf16x8(raw[0]);
 #pragma unroll
-      for (int nn = 0; nn < 6; nn++) {
-        const unsigned char* src = wt + (32 * ks2 + 8 * kg + (l16 >> 1)) * WS + cw0 + 16 * nn + (l16 & 1) * 8;
-        intx2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(lds_u8*)src);
-        floatx2 f01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, false), f23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.x, true);
-        floatx2 f45 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, false), f67 = __builtin_amdgcn_cvt_pk_f32_fp8(raw.y, true);
-        bf16x8 wb = {(__bf16)f01.x, (__bf16)f01.y, (__bf16)f23.x, (__bf16)f23.y,
-                     (__bf16)f45.x, (__bf16)f45.y, (__bf16)f67.x, (__bf16)f67.y};
+      for (int s = 0; s < 12; s++) {
+        const int ks2 = s / 6, nn = s - ks2 * 6;
+        if (s + 2 < 12) raw[(s + 2) % 3] = lds_tr8(wsrc + ((s + 2) / 6) * 32 * WS + ((s + 2) % 6) * 16);
+        if (s < 4) {   // second K step's G^T operands, two per step
+          ga[1][2 * s] = *(const bf16x8*)(gsrc + 16 * (2 * s) * GT_S + 64);
+          ga[1][2 * s + 1] = *(const bf16x8*)(gsrc + 16 * (2 * s + 1) * GT_S + 64);
+        }
+        SCHED_FENCE();
 #pragma unroll
-        for (int mb = 0; mb < 8; mb++)
-          acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb, acc2[mb][nn], 0, 0, 0);
+        for (int mb = 0; mb < 8; mb++) {
+          acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[ks2][mb], wb[s & 1], acc2[mb][nn], 0, 0, 0);
+          if (mb == 1 && s + 1 < 12) wb[(s + 1) & 1] = fp8x8_to_bf16x8(raw[(s + 1) % 3]);
+          if (mb == 1) SCHED_FENCE();
+        }
+        SCHED_FENCE();
       }
     }
 
-    // ---- 4+5. A^T[96 x 64] = X^T G^T, then the update of this wavefront's 96 features, in LDS
-#pragma unroll 1
-    for (int half = 0; half < 2; half++) {
-      floatx4 acc3[3][4];
+    // ---- 4+5. A^T[96 x 64] = X^T G^T in six 16-feature groups; the update of group g-1 (VALU, in LDS) is
+    //           issued between the MFMAs of group g.  G operands stay in registers for all six groups.
+    {
+      bf16x8 bg[4][4];   // [ks][nb]
 #pragma unroll
-      for (int a = 0; a < 3; a++)
+      for (int ks = 0; ks < 4; ks++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) acc3[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int nb = 0; nb < 4; nb++) bg[ks][nb] = *(const bf16x8*)(gl + (16 * nb + l16) * GL_S + ks * 64 + kg * 16);
+      const bf16x8* xsrc = p.xt + (size_t)cb0 * 4 * 64 + lane;
+      bf16x8 ax[2][4];
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) {
-        bf16x8 bg[4];
+      for (int ks = 0; ks < 4; ks++) ax[0][ks] = xsrc[ks * 64];
+      floatx4 acc3[2][4];
+      unsigned char* wrow = wt + l16 * WS + cw0 + 4 * kg;
+      const unsigned grow0 = (unsigned)(c * p.rows_per_chunk + row0 + l16);
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) bg[nb] = *(const bf16x8*)(gl + (16 * nb + l16) * GL_S + ks * 64 + kg * 16);
+      for (int cg = 0; cg <= 6; cg++) {
+        const int cur = cg & 1, prev = cur ^ 1;
+        if (cg < 6) {
+          if (cg + 1 < 6) {
 #pragma unroll
-        for (int m3 = 0; m3 < 3; m3++) {
-          bf16x8 ax = p.xt[(size_t)((cb0 + half * 3 + m3) * 4 + ks) * 64 + lane];
+            for (int ks = 0; ks < 4; ks++) ax[prev][ks] = xsrc[((cg + 1) * 4 + ks) * 64];
+          }
 #pragma unroll
-          for (int nb = 0; nb < 4; nb++)
-            acc3[m3][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bg[nb], acc3[m3][nb], 0, 0, 0);
+          for (int nb = 0; nb < 4; nb++) acc3[cur][nb] = floatx4{0.f, 0.f, 0.f, 0.f};
         }
-      }
+        unsigned wq[4];
+        if (cg > 0 && !(XMC_DBG_SKIP & 16)) {
 #pragma unroll
-      for (int m3 = 0; m3 < 3; m3++) {
+          for (int nb = 0; nb < 4; nb++) wq[nb] = *(const unsigned*)(wrow + 16 * nb * WS + 16 * (cg - 1));
+        }
+        SCHED_FENCE();
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++) {
-          const int row = 16 * nb + l16;
-          const int col = cw0 + 16 * (half * 3 + m3) + 4 * kg;
-          unsigned* wp = (unsigned*)(wt + row * WS + col);
-          unsigned wq = *wp;
-          floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq, true);
-          floatx4 a = acc3[m3][nb];
-          float t0 = __builtin_fmaf(-p.lr_eff, a[0], w01.x), t1 = __builtin_fmaf(-p.lr_eff, a[1], w01.y);
-          float t2 = __builtin_fmaf(-p.lr_eff, a[2], w23.x), t3 = __builtin_fmaf(-p.lr_eff, a[3], w23.y);
-          *wp = round4<MODE>(t0, t1, t2, t3, (unsigned)(row0 + row), (unsigned)(c * p.rows_per_chunk + row0 + row),
-                             (unsigned)col, seed);
+        for (int q = 0; q < 4; q++) {   // q = K step for the MFMAs, = row block for the update
+          if (cg < 6 && !(XMC_DBG_SKIP & 8)) {
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++)
+              acc3[cur][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[cur][q], bg[q][nb], acc3[cur][nb], 0, 0, 0);
+          }
+          if (cg > 0 && !(XMC_DBG_SKIP & 16)) {
+            const int nb = q;
+            floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq[nb], false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wq[nb], true);
+            floatx4 a = acc3[prev][nb];
+            float t0 = __builtin_fmaf(-p.lr_eff, a[0], w01.x), t1 = __builtin_fmaf(-p.lr_eff, a[1], w01.y);
+            float t2 = __builtin_fmaf(-p.lr_eff, a[2], w23.x), t3 = __builtin_fmaf(-p.lr_eff, a[3], w23.y);
+            const unsigned col = (unsigned)(cw0 + 16 * (cg - 1) + 4 * kg);
+            *(unsigned*)(wrow + 16 * nb * WS + 16 * (cg - 1)) =
+                round4<MODE>(t0, t1, t2, t3, (unsigned)(row0 + 16 * nb + l16), grow0 + 16 * nb, col, seed);
+          }
+          SCHED_FENCE();
         }
       }
     }
+    // logits operands of the first two K steps of the next tile
+    xqb[0][0] = xqw[0]; xqb[0][1] = xqw[6 * 64];
+    xqb[1][0] = xqw[1 * 64]; xqb[1][1] = xqw[7 * 64];
     __builtin_amdgcn_s_waitcnt(0);   // next tile has landed in LDS (this thread's part)
     __syncthreads();
     if (tid == 0) __hip_atomic_store(flag_mine, it + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // the partner must hold this tile before its rows are overwritten
-    for (int spin = 0; seen < it + 1; spin++) {
+    for (int spin = 0; seen < it + 1 && !(XMC_DBG_SKIP & 128); spin++) {
       if (spin >= SPIN_LIMIT) { p.flags[2 * npairs] = 1; break; }
       __builtin_amdgcn_s_sleep(2);
       seen = __hip_atomic_load(flag_other, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -259,7 +332,7 @@ __global__ __launch_bounds__(NT, 1) void fp8_step_kernel(const StepParams p) {
     for (int s = 0; s < 6; s++) {
       int ch = s * NT + tid;
       int row = ch / 24, cc = ch - row * 24;
-      if (row < rows_valid) {
+      if (row < rows_valid && !(XMC_DBG_SKIP & 64)) {
         uint4 v = *(const uint4*)(wt + row * WS + HALF * h + cc * 16);
         *(uint4*)(gchunk + (size_t)(row0 + row) * D + HALF * h + cc * 16) = v;
       }

@@ -74,6 +74,11 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Benchmarking aid (no counterpart in the reference): the next xmc_fp8_step call records these two HIP events
+ * (hipEvent_t, created by the caller) immediately before and after its fused step kernel, on the call's stream,
+ * then forgets them.  Pass nulls to cancel. */
+int xmc_profile_events(void* start_event, void* stop_event);
+
 /* Reads back the error word a step leaves in the workspace (non-zero: a workgroup gave up waiting for its
  * partner).  Synchronises the stream; meant for tests and debugging, not for the training loop. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);

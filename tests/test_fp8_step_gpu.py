@@ -38,8 +38,13 @@ def check_rtn(case, device, **kw):
     scale = np.abs(ref_gx).max()
     assert np.abs(gx - ref_gx).max() <= 1e-2 * scale
     assert np.abs(gx - ref_gx).max() <= 1e-3 * scale      # fp32 reassociation plus a few 1-ulp flips of bf16 G
-    big = np.abs(ref_gx) > 1e-2 * scale
-    assert H.bf16_ulp_distance(gb, ref_gb)[big].max() <= 1
+    # grad_input is the round-to-nearest-even bf16 image of the fp32 accumulator ...
+    assert np.array_equal(C.bf16_bits(gb), C.bf16_bits(C.bf16_round(gx)))
+    # ... and within 1 bf16 ulp of the oracle's wherever the two accumulators agree to a quarter ulp
+    ulp = np.abs(ref_gb) * 2.0 ** -8 + 1e-30
+    close = np.abs(gx - ref_gx) < 0.25 * ulp
+    assert close.mean() > 0.5
+    assert H.bf16_ulp_distance(gb, ref_gb)[close].max() <= 1
     return mism / total
 
 
