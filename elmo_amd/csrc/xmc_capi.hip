@@ -2,6 +2,8 @@
 // Declarations and the reference interfaces they replace: include/elmo_xmc.h.
 #include "../../include/elmo_xmc.h"
 #include "xmc_fp8_step.hip"
+#include "xmc_fp8_quad.hip"
+#include <stdlib.h>
 
 using namespace xmc;
 
@@ -22,6 +24,9 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
     (void)hipFuncSetAttribute((const void*)sort_keys_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
   }
@@ -101,40 +106,77 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
 
   (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
-  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
-                                                              (unsigned short*)(ws + WS_XT));
   if (n_pad > 0)
     sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
                                                                 tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
-  StepParams p;
-  for (int c = 0; c < MAX_CHUNKS; c++) {
-    p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
-    p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+  static const bool use_pair = !(getenv("XMC_KERNEL") && !__builtin_strcmp(getenv("XMC_KERNEL"), "quad"));
+  if (use_pair) {
+    prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
+                                                                (unsigned short*)(ws + WS_XT));
+    StepParams p;
+    for (int c = 0; c < MAX_CHUNKS; c++) {
+      p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
+      p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+    }
+    p.num_chunks = num_chunks;
+    p.rows_per_chunk = rows_per_chunk;
+    p.tiles_per_chunk = tiles_per_chunk;
+    p.num_tiles = num_tiles;
+    p.xq = ws + WS_XQ;
+    p.xt = (const bf16x8*)(ws + WS_XT);
+    p.keys = (const unsigned*)(ws + WS_KEYS);
+    p.tile_ptr = (const int*)(ws + WS_TILEPTR);
+    p.partial = (floatx4*)(ws + WS_PARTIAL);
+    p.flags = (int*)(ws + WS_FLAGS);
+    p.zscale = scale_w * scale_x;
+    p.lr_eff = lr / scale_w;
+    p.batch = batch;
+    if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
+    switch (round_mode) {
+      case XMC_ROUND_RTN: fp8_step_kernel<ROUND_RTN><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+      case XMC_ROUND_SR_PHILOX: fp8_step_kernel<ROUND_SR_PHILOX><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+      default: fp8_step_kernel<ROUND_SR_FAST><<<grid, NT, LDS_BYTES, stream>>>(p); break;
+    }
+    if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
+    g_prof_start = g_prof_stop = nullptr;
+    reduce_gx_kernel<<<96, NT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), grid, scale_w, grad_x_f32,
+                                           (unsigned short*)grad_x_bf16, batch);
+  } else {
+    prep_x_quad_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x,
+                                                                     ws + WS_XQ, (unsigned short*)(ws + WS_XT));
+    QuadParams p;
+    for (int c = 0; c < MAX_CHUNKS; c++) {
+      p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
+      p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+    }
+    p.num_chunks = num_chunks;
+    p.rows_per_chunk = rows_per_chunk;
+    p.tiles_per_chunk = tiles_per_chunk;
+    p.num_tiles = num_tiles;
+    p.xq = ws + WS_XQ;
+    p.xt = (const bf16x8*)(ws + WS_XT);
+    p.keys = (const unsigned*)(ws + WS_KEYS);
+    p.tile_ptr = (const int*)(ws + WS_TILEPTR);
+    p.partial = (floatx4*)(ws + WS_PARTIAL);
+    p.exch = ws + WS_EXCH;
+    p.flags = (int*)(ws + WS_FLAGS);
+    p.zscale = scale_w * scale_x;
+    p.lr_eff = lr / scale_w;
+    p.batch = batch;
+    const int qgrid = grid / 32 * 32;   // whole quads on every XCD
+    if (qgrid < 32) return XMC_ERR_DEVICE;
+    if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
+    switch (round_mode) {
+      case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
+      case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
+      default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
+    }
+    if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
+    g_prof_start = g_prof_stop = nullptr;
+    reduce_gx_quad_kernel<<<48, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+                                                 (unsigned short*)grad_x_bf16, batch);
   }
-  p.num_chunks = num_chunks;
-  p.rows_per_chunk = rows_per_chunk;
-  p.tiles_per_chunk = tiles_per_chunk;
-  p.num_tiles = num_tiles;
-  p.xq = ws + WS_XQ;
-  p.xt = (const bf16x8*)(ws + WS_XT);
-  p.keys = (const unsigned*)(ws + WS_KEYS);
-  p.tile_ptr = (const int*)(ws + WS_TILEPTR);
-  p.partial = (floatx4*)(ws + WS_PARTIAL);
-  p.flags = (int*)(ws + WS_FLAGS);
-  p.zscale = scale_w * scale_x;
-  p.lr_eff = lr / scale_w;
-  p.batch = batch;
-  if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
-  switch (round_mode) {
-    case XMC_ROUND_RTN: fp8_step_kernel<ROUND_RTN><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-    case XMC_ROUND_SR_PHILOX: fp8_step_kernel<ROUND_SR_PHILOX><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-    default: fp8_step_kernel<ROUND_SR_FAST><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-  }
-  if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
-  g_prof_start = g_prof_stop = nullptr;
-  reduce_gx_kernel<<<96, NT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), grid, scale_w, grad_x_f32,
-                                         (unsigned short*)grad_x_bf16, batch);
   return launch_status();
 }
 

@@ -85,8 +85,10 @@ __device__ __forceinline__ void issue_tile_load(const unsigned char* gtile, int 
       row = row < last_row ? row : last_row;
       c = c < 47 ? c : 47;
       const unsigned char* g = gtile + (size_t)row * D + c * 16;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                       (__attribute__((address_space(3))) void*)(dst + (s * NT + (tid & ~63)) * 16), 16, 0, 0);
+      // inline assembly on purpose: the compiler would order every later LDS access behind a direct-to-LDS
+      // load it knows about; completion is enforced by hand (s_waitcnt vmcnt(0) + barrier) before use
+      const unsigned ldsoff = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(dst + (s * NT + (tid & ~63)) * 16));
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsoff), "v"(g) : "memory", "m0");
     }
   }
 }
