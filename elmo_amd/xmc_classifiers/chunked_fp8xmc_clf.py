@@ -1,0 +1,135 @@
+"""FP8 chunked extreme-classifier layer on the MI355X kernels.
+
+Mirror of the reference's Fp8XMCBCEChunkedLayer (src/xmc_classifiers/chunked_fp8xmc_clf.py): same constructor
+argument, methods (`xfc_forward`, `xfc_forward_backward`, `filter_non_local_inds`), attributes (`xfc_weight`
+ParameterList of e4m3fn chunks, `grad_input`, `_dtype`, `num_labels`, `num_labels_i`, `iteration`, `loss`) and
+error convention (AssertionError for shape / layout / device problems), so src/model.py and src/runner.py can
+use it unchanged.  The per-chunk Python loop of the reference is replaced by ONE call into the C ABI that
+covers all chunks; there is no CPU or PyTorch fallback.
+
+Configuration read (attribute style, OmegaConf not required):
+  environment.device, data.num_labels, model.xmc.num_chunks, model.xmc.input_features,
+  training.xmc.simulated_fp8
+Optional, not in the reference (all default to the reference's behaviour):
+  training.xmc.rounding   "sr_fast" (default) | "sr_philox" | "rtn"
+        sr_philox reproduces the reference's bit recipe (Philox word per element, fuse_kernel.py:29-36);
+        sr_fast rounds stochastically with the hardware converter and a counter hash: unbiased on the whole
+        e4m3 grid (subnormals included), not bit-identical to the reference's random stream
+  training.xmc.scale_w, training.xmc.scale_x   per-tensor scales (reference: 1.0, 1.0)
+"""
+import torch
+from torch import nn
+
+from .. import ops
+
+dtype_map = {'float16': torch.float16, 'bfloat16': torch.bfloat16, 'float32': torch.float32,
+             'float8': torch.float8_e4m3fn}
+
+
+def _opt(node, name, default):
+    try:
+        v = getattr(node, name)
+    except Exception:
+        return default
+    return default if v is None else v
+
+
+class Fp8XMCBCEChunkedLayer(nn.Module):
+    '''
+    Chunked FP8 XMC classifier
+    '''
+
+    def __init__(self, cfg):
+        super(Fp8XMCBCEChunkedLayer, self).__init__()
+        self.cfg = cfg
+        self.device = torch.device(cfg.environment.device)
+        self._dtype = torch.float8_e4m3fn
+        self.fake_fp8_matmul = cfg.training.xmc.simulated_fp8
+        self.num_chunks = self.cfg.model.xmc.num_chunks
+        # reference padding rule (chunked_fp8xmc_clf.py:26): always adds between 1 and 16*num_chunks rows
+        self.num_labels = cfg.data.num_labels + 16 * self.num_chunks - cfg.data.num_labels % (16 * self.num_chunks)
+        self.num_labels_i = self.num_labels // self.num_chunks
+        assert self.num_labels_i % 16 == 0
+        features = cfg.model.xmc.input_features
+        assert features == ops.FEATURES, f"the gfx950 kernels are built for {ops.FEATURES} input features"
+        assert self.device.type == "cuda", "Fp8XMCBCEChunkedLayer needs a GPU device: there is no CPU path"
+        assert not self.fake_fp8_matmul, "training.xmc.simulated_fp8 is not implemented by this build"
+
+        # same initialisation as the reference (:29-32): xavier-uniform on the padded fp32 matrix, cast per chunk
+        xfc_weight = torch.empty(self.num_labels, features, dtype=torch.float32)
+        nn.init.xavier_uniform_(xfc_weight)
+        self.xfc_weight = nn.ParameterList([
+            nn.Parameter(xfc_weight[i * self.num_labels_i:(i + 1) * self.num_labels_i].to(torch.float8_e4m3fn)
+                         .to(self.device).contiguous(), requires_grad=False)
+            for i in range(self.num_chunks)])
+        del xfc_weight
+        n_labels = 0
+        for i in range(self.num_chunks):
+            n_labels += self.xfc_weight[i].shape[0]
+            assert self.xfc_weight[i].shape[0] == self.num_labels_i
+        assert n_labels == self.num_labels
+
+        self.rounding = _opt(cfg.training.xmc, "rounding", "sr_fast")
+        assert self.rounding in ("sr_fast", "sr_philox", "rtn")
+        self.scale_w = float(_opt(cfg.training.xmc, "scale_w", 1.0))
+        self.scale_x = float(_opt(cfg.training.xmc, "scale_x", 1.0))
+        self.block_size = 16
+        self.loss = torch.tensor(0.0, device=self.device)
+        self.iteration = 0
+        self.grad_input = None
+        # all scratch memory of the step comes from the torch allocator (so that max_memory_allocated sees it)
+        self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
+
+    def _chunks(self):
+        return [w.data for w in self.xfc_weight]
+
+    @torch.no_grad()
+    def xfc_forward(self, embed):
+        '''
+        Mainly used during inference: logits [B, cfg.data.num_labels] in bf16 (padding rows dropped).
+        '''
+        assert embed.is_cuda and embed.dim() == 2
+        return ops.fp8_forward(self._chunks(), embed, self.cfg.data.num_labels, self.scale_w, self.scale_x,
+                               self._workspace)
+
+    @torch.no_grad()
+    def _compute_loss(self, outlogit, rows, cols):
+        '''
+        BCE-with-logits summed over a dense logit block (reference :62-78; never reached in training because
+        the training loop always passes skip_loss=True).
+        '''
+        z = outlogit.float()
+        loss = z.clamp(min=0.0).sum() - z[rows, cols].sum() + torch.log1p(torch.exp(-z.abs())).sum()
+        return loss.item()
+
+    @torch.no_grad()
+    def xfc_forward_backward(self, embed, labels, xmc_lr, skip_loss=True):
+        '''
+        Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
+        Args:
+            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 128.
+            labels: Positive labels in sparse format, int32 [Nb, 2] = (row in batch, label id).
+            xmc_lr: list of learning rates, only [0] is used.
+            skip_loss: ignored, as in the reference's FP8 layer; the return value is 0.
+        '''
+        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
+        assert embed.shape[0] % 16 == 0 and embed.shape[0] <= ops.MAX_BATCH, \
+            "batch must be a multiple of 16 and at most 128 (the reference data loader uses drop_last)"
+        assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
+        x = embed.detach()
+        if x.dtype != torch.bfloat16:
+            x = x.to(torch.bfloat16)
+        x = x.contiguous()
+        lab = labels if labels.dtype == torch.int32 else labels.to(torch.int32)
+        lab = lab.contiguous()
+        loss = 0
+        # one seed per chunk from the global CPU generator, exactly as the reference draws them (:113)
+        seeds = [torch.randint(0, 1000000, (1,)).item() for _ in range(self.num_chunks)]
+        self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
+                                       scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
+        self.iteration += 1
+        return loss
+
+    def filter_non_local_inds(self, rows, cols, start, end):
+        mask = (cols >= start) & (cols < end)
+        return rows[mask], cols[mask] - start

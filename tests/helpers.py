@@ -53,3 +53,14 @@ def chunks_to_numpy(chunks):
 def bf16_tensor_to_f32_numpy(t):
     import torch
     return t.float().cpu().numpy()
+
+
+def assert_bf16_close(got, ref, floor_rel=5e-5, min_equal=0.99):
+    """bf16 values agree to 1 ulp, except next to zero where cancellation in the fp32 accumulator dominates: there
+    the difference must stay below floor_rel * max|ref|.  Most entries must be identical."""
+    got = np.asarray(got, dtype=np.float32)
+    ref = np.asarray(ref, dtype=np.float32)
+    ulp = np.abs(ref) * 2.0 ** -7
+    tol = np.maximum(ulp, floor_rel * np.abs(ref).max())
+    assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) / tol))
+    assert np.mean(got == ref) >= min_equal, float(np.mean(got == ref))

@@ -1,0 +1,82 @@
+"""The headline workload at its full size (670 091 labels, 11 chunks, batch 128), checked through properties that
+do not need the whole oracle: sampled label rows against the oracle (the update of a row depends only on that
+row, X and the positives), lr = 0 leaves every weight byte unchanged, grad_X against an fp32 library GEMM, and
+positives change exactly the rows they name."""
+import numpy as np
+import pytest
+
+import helpers as H
+from elmo_amd import synth
+from oracle import codecs as C
+from oracle import step as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def big(gpu):
+    import torch
+    cfg = synth.CONFIGS["cfg2_fp8_670k"]
+    nc = cfg.num_chunks
+    L_pad = O.fp8_padded_labels(cfg.num_labels, nc)
+    rows = L_pad // nc
+    gen = torch.Generator(device=gpu).manual_seed(cfg.seed)
+    chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.02).to(torch.float8_e4m3fn) for _ in range(nc)]
+    x_np = synth.make_x(cfg.batch, 768, cfg.seed)
+    labels_np = synth.make_labels(cfg.batch, cfg.num_labels, cfg.pos_mean, cfg.zipf_s, cfg.seed)
+    x = torch.from_numpy(x_np).to(gpu).to(torch.bfloat16)
+    labels = torch.from_numpy(labels_np).to(gpu)
+    return dict(cfg=cfg, nc=nc, rows=rows, chunks=chunks, x=x, labels=labels, x_np=x_np, labels_np=labels_np)
+
+
+def test_lr_zero_is_identity_and_gradx_matches_library_gemm(gpu, big):
+    import torch
+    from elmo_amd import ops
+    before = [c.view(torch.uint8).clone() for c in big["chunks"]]
+    ws = ops.alloc_workspace(big["nc"], big["rows"], gpu)
+    g, gf = ops.fp8_step(big["chunks"], big["x"], big["labels"], 0.0, round_mode="rtn", workspace=ws, want_f32=True)
+    assert ops.step_error_word(ws, big["nc"], big["rows"]) == 0
+    for a, c in zip(before, big["chunks"]):
+        b = c.view(torch.uint8)
+        same = (a == b) | (((a | b) & 0x7F) == 0)          # +0 and -0 are the same weight
+        assert bool(same.all())
+    # grad_X = G^T W with G from bf16 logits of the FP8-quantised X: fp32 library GEMMs on the same device
+    xq = big["x"].to(torch.float8_e4m3fn).float()
+    ref = torch.zeros(128, 768, device=gpu, dtype=torch.float64)
+    lab = big["labels"].long()
+    for c, wc in enumerate(big["chunks"]):
+        w = wc.float()
+        z = (w @ xq.t()).to(torch.bfloat16).float()
+        s = torch.sigmoid(z).to(torch.bfloat16)
+        sel = (lab[:, 1] >= c * big["rows"]) & (lab[:, 1] < (c + 1) * big["rows"])
+        s[lab[sel, 1] - c * big["rows"], lab[sel, 0]] -= 1.0
+        ref += (s.double().t() @ w.double())
+    ref = ref.float()
+    scale = ref.abs().max().item()
+    assert (gf - ref).abs().max().item() <= 1e-2 * scale
+    assert (gf - ref).abs().max().item() <= 2e-3 * scale
+    assert torch.equal(g.view(torch.int16), gf.to(torch.bfloat16).view(torch.int16))
+
+
+def test_sampled_rows_match_oracle_after_a_real_step(gpu, big):
+    import torch
+    from elmo_amd import ops
+    nc, rows = big["nc"], big["rows"]
+    rng = np.random.default_rng(0)
+    # rows around tile and chunk boundaries, the head labels (where the positives are), and random ones
+    pos_rows = np.unique(big["labels_np"][:, 1])
+    sample = np.unique(np.concatenate([np.arange(0, 130), pos_rows[:200], [rows - 1, rows, rows + 1, 2 * rows - 1, nc * rows - 1],
+                                       rng.integers(0, nc * rows, 400)]))
+    before = {int(r): big["chunks"][r // rows][r % rows].view(torch.uint8).cpu().numpy().copy() for r in sample}
+    ws = ops.alloc_workspace(nc, rows, gpu)
+    ops.fp8_step(big["chunks"], big["x"], big["labels"], 0.05, round_mode="rtn", workspace=ws)
+    assert ops.step_error_word(ws, nc, rows) == 0
+    w_old = np.stack([before[int(r)] for r in sample])
+    # oracle on the sampled rows only: remap the positives that name a sampled row
+    remap = {int(r): i for i, r in enumerate(sample)}
+    lab = np.array([(b, remap[int(l)]) for b, l in big["labels_np"] if int(l) in remap], dtype=np.int32).reshape(-1, 2)
+    ref_codes, _, _ = O.fp8_step([w_old], big["x_np"], lab, 0.05, sr_mode="rtn")
+    got = np.stack([big["chunks"][r // rows][r % rows].view(torch.uint8).cpu().numpy() for r in sample])
+    d = H.e4m3_ulp_distance(got, ref_codes[0])
+    assert d.max() <= 1 and np.mean(d != 0) < 2e-3
+    assert np.mean(got != w_old) > 0.3                       # the step really changed the weights

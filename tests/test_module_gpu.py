@@ -1,0 +1,124 @@
+"""The drop-in classifier module driven exactly as the reference's training loop and evaluator drive it
+(src/runner.py:139-157, src/evaluate.py:153-159), with a stub encoder in place of the transformer."""
+import io
+
+import numpy as np
+import pytest
+
+import helpers as H
+from test_host_cpu import make_cfg
+from oracle import codecs as C
+from oracle import step as O
+
+pytestmark = pytest.mark.gpu
+
+
+def build(gpu, num_labels=1000, num_chunks=2, **extra):
+    import torch
+    from xmc_classifiers.chunked_fp8xmc_clf import Fp8XMCBCEChunkedLayer
+    torch.manual_seed(0)
+    return Fp8XMCBCEChunkedLayer(make_cfg("cuda:0", num_labels, num_chunks, **extra))
+
+
+def test_construction_matches_reference_layout(gpu):
+    import torch
+    xfc = build(gpu, 1000, 2)
+    assert xfc.num_labels == 1000 + 32 - 1000 % 32 == 1024 and xfc.num_labels_i == 512      # padding rule
+    assert xfc._dtype == torch.float8_e4m3fn and len(xfc.xfc_weight) == 2
+    assert all(w.dtype == torch.float8_e4m3fn and w.shape == (512, 768) and not w.requires_grad and w.is_cuda
+               for w in xfc.xfc_weight)
+    assert sorted(xfc.state_dict().keys()) == ["xfc_weight.0", "xfc_weight.1"]
+    # xavier-uniform bound sqrt(6 / (L_pad + d)) before the cast: every code decodes inside it (plus rounding)
+    bound = np.sqrt(6.0 / (1024 + 768))
+    w = C.e4m3_decode(xfc.xfc_weight[0].view(torch.uint8).cpu().numpy())
+    assert np.abs(w).max() <= bound * 1.07 and np.abs(w).max() > bound * 0.8
+    xfc2 = build(gpu, 1024, 2)
+    assert xfc2.num_labels == 1056                     # already aligned: a full extra group of 16 * num_chunks
+
+
+def test_training_call_contract(gpu):
+    import torch
+    xfc = build(gpu, 1000, 2, rounding="rtn")
+    enc = torch.nn.Linear(768, 768, bias=False).to(gpu).to(torch.bfloat16)
+    torch.manual_seed(1)
+    tokens = torch.randn(32, 768, device=gpu, dtype=torch.bfloat16)
+    labels = torch.tensor([[0, 3], [0, 999], [5, 17], [31, 500], [31, 500]], dtype=torch.int32, device=gpu)
+    ptrs = [w.data_ptr() for w in xfc.xfc_weight]
+    before = [w.view(torch.uint8).clone() for w in xfc.xfc_weight]
+
+    out = enc(tokens)                                   # has grad_fn
+    out_copy = out.detach().clone()
+    grad_fn = out.grad_fn
+    loss = xfc.xfc_forward_backward(out, labels, [0.05], skip_loss=True)
+    assert loss == 0 and xfc.iteration == 1
+    assert torch.equal(out.detach().view(torch.int16), out_copy.view(torch.int16)) and out.grad_fn is grad_fn
+    g = xfc.grad_input
+    assert g.shape == (32, 768) and g.dtype == out.dtype and g.is_cuda
+    g[0:32, :].div_(2)                                  # runner.py:155 (gradient accumulation)
+    out.backward(g[0:32, :])                            # runner.py:157
+    expect = (g.float().t() @ tokens.float())           # closed form of the stub's weight gradient
+    assert torch.allclose(enc.weight.grad.float(), expect, rtol=2e-2, atol=2e-2 * expect.abs().max().item())
+    # weights were updated in place
+    assert [w.data_ptr() for w in xfc.xfc_weight] == ptrs
+    assert any(not torch.equal(a, w.view(torch.uint8)) for a, w in zip(before, xfc.xfc_weight))
+    # parity of this exact call with the oracle
+    chunks_np = [b.cpu().numpy() for b in before]
+    x_np = out_copy.float().cpu().numpy()
+    ref_codes, ref_gx, ref_gb = O.fp8_step(chunks_np, x_np, labels.cpu().numpy(), 0.05, sr_mode="rtn")
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        assert H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r).max() <= 1
+    assert np.abs(g.float().cpu().numpy() * 2 - ref_gb).max() <= 2e-2 * np.abs(ref_gb).max()
+
+
+def test_default_rounding_draws_seeds_from_the_global_cpu_generator(gpu):
+    import torch
+    xfc = build(gpu, 500, 3)
+    assert xfc.rounding == "sr_fast"
+    x = torch.randn(16, 768, device=gpu).to(torch.bfloat16)
+    labels = torch.zeros((0, 2), dtype=torch.int32, device=gpu)
+    torch.manual_seed(123)
+    expected_next = None
+    xfc.xfc_forward_backward(x, labels, [0.05])
+    after = torch.randint(0, 1000000, (1,)).item()
+    torch.manual_seed(123)
+    for _ in range(3):                                   # one draw per chunk, as chunked_fp8xmc_clf.py:113
+        torch.randint(0, 1000000, (1,)).item()
+    assert torch.randint(0, 1000000, (1,)).item() == after
+
+
+def test_evaluator_contract_and_checkpoint_roundtrip(gpu):
+    import torch
+    xfc = build(gpu, 1000, 2)
+    torch.manual_seed(2)
+    embed = torch.randn(40, 768, device=gpu).to(torch.bfloat16)
+    logits = xfc.xfc_forward(embed.to(xfc._dtype))       # evaluate.py:155-158
+    assert logits.shape == (40, 1000) and logits.dtype == torch.bfloat16
+    vals, idx = torch.topk(logits, k=5)                  # evaluate.py:159
+    chunks_np = [w.view(torch.uint8).cpu().numpy() for w in xfc.xfc_weight]
+    ref = O.fp8_forward(chunks_np, embed.float().cpu().numpy(), 1000)
+    H.assert_bf16_close(logits.float().cpu().numpy(), ref)
+    ref_top = np.argsort(-ref, axis=1, kind="stable")[:, :5]
+    assert np.mean(np.sort(ref_top, axis=1) == np.sort(idx.cpu().numpy(), axis=1)) > 0.97
+    # runner.py:246 pickles xfc.xfc_weight with torch.save; :257 assigns it back
+    buf = io.BytesIO()
+    torch.save({"xfc_weight": xfc.xfc_weight, "model": xfc.state_dict()}, buf)
+    buf.seek(0)
+    ck = torch.load(buf, weights_only=False)
+    for a, b in zip(ck["xfc_weight"], xfc.xfc_weight):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    xfc.load_state_dict(ck["model"])
+
+
+def test_error_convention(gpu):
+    import torch
+    xfc = build(gpu, 1000, 2)
+    labels = torch.zeros((0, 2), dtype=torch.int32, device=gpu)
+    with pytest.raises(AssertionError):
+        xfc.xfc_forward_backward(torch.randn(17, 768, device=gpu).to(torch.bfloat16), labels, [0.05])
+    with pytest.raises(AssertionError):
+        xfc.xfc_forward_backward(torch.randn(16, 512, device=gpu).to(torch.bfloat16), labels, [0.05])
+    with pytest.raises(AssertionError):
+        xfc.xfc_forward_backward(torch.randn(16, 768).to(torch.bfloat16), labels, [0.05])
+    with pytest.raises(AssertionError):
+        build(gpu, 1000, 2, ) if False else __import__("xmc_classifiers.chunked_fp8xmc_clf", fromlist=["x"]).Fp8XMCBCEChunkedLayer(
+            make_cfg("cuda:0", 1000, 2, simulated=True))
