@@ -24,9 +24,9 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES + XMC_DBG_TIMING * 6144);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
     (void)hipFuncSetAttribute((const void*)sort_keys_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
   }
@@ -168,13 +168,13 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     if (qgrid < 32) return XMC_ERR_DEVICE;
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
     switch (round_mode) {
-      case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
-      case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
-      default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES + XMC_DBG_TIMING * 6144, stream>>>(p); break;
+      case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+      case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+      default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
-    reduce_gx_quad_kernel<<<48, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+    reduce_gx_quad_kernel<<<96, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
                                                  (unsigned short*)grad_x_bf16, batch);
   }
   return launch_status();
