@@ -66,6 +66,8 @@ def main():
     ap.add_argument("--config", default="cfg2_fp8_670k")
     ap.add_argument("--round", default="sr_fast", choices=["sr_fast", "sr_philox", "rtn"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="only launch the library's plain copy kernel over MIB MiB five times (counter calibration) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the classifier step on ONE GPU; --gpus > 1 is not supported "
@@ -83,6 +85,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = _lib.load()
+    if args.copy_calibration > 0:
+        nbytes = args.copy_calibration << 20
+        src = torch.full((nbytes,), 3, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(5):
+            _lib.check(lib.xmc_copy_probe(dst.data_ptr(), src.data_ptr(), nbytes, stream), "xmc_copy_probe")
+        torch.cuda.synchronize()
+        assert bool((dst == 3).all())
+        print(json.dumps({"copy_probe_kernel": {"bytes_read": nbytes, "bytes_written": nbytes, "launches": 5}}))
+        return
     nc = cfg.num_chunks
     L_pad = padded_labels(cfg.num_labels, nc)
     rows = L_pad // nc

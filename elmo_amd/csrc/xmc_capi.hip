@@ -54,6 +54,11 @@ int check_common(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   return XMC_OK;
 }
 
+// plain 16-byte-per-lane copy: the known-size reference against which memory counters are calibrated
+__global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
 int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
 
 }  // namespace
@@ -80,7 +85,7 @@ const char* xmc_error_string(int status) {
 size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk) {
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
   size_t tiles = (size_t)num_chunks * ((rows_per_chunk + TL - 1) / TL);
-  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256;
+  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256 + tiles * 32;   // tile_ptr, then 32-byte tile descriptors
 }
 
 int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
@@ -160,12 +165,15 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.tile_ptr = (const int*)(ws + WS_TILEPTR);
     p.partial = (floatx4*)(ws + WS_PARTIAL);
     p.exch = ws + WS_EXCH;
+    uint4* desc = (uint4*)(ws + WS_TILEPTR + ((size_t)(num_tiles + 1) * 4 + 255) / 256 * 256);
+    p.desc = desc;
     p.flags = (int*)(ws + WS_FLAGS);
     p.zscale = scale_w * scale_x;
     p.lr_eff = lr / scale_w;
     p.batch = batch;
     const int qgrid = grid / 32 * 32;   // whole quads on every XCD
     if (qgrid < 32) return XMC_ERR_DEVICE;
+    tile_desc_kernel<<<(num_tiles + 255) / 256, 256, 0, stream>>>(p, desc);
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
     switch (round_mode) {
       case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
@@ -207,6 +215,14 @@ int xmc_profile_events(void* start_event, void* stop_event) {
   g_prof_start = (hipEvent_t)start_event;
   g_prof_stop = (hipEvent_t)stop_event;
   return XMC_OK;
+}
+
+int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream_) {
+  if (!dst || !src) return XMC_ERR_NULL;
+  if (!aligned16(dst) || !aligned16(src) || bytes % 16 != 0) return XMC_ERR_ALIGN;
+  if (bytes == 0) return XMC_OK;
+  copy_probe_kernel<<<2048, 256, 0, (hipStream_t)stream_>>>((const uint4*)src, (uint4*)dst, bytes / 16);
+  return launch_status();
 }
 
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream_) {

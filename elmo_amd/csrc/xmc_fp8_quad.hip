@@ -3,19 +3,22 @@
 // Work unit = a tile of 64 consecutive label rows of one chunk (64 x 768 e4m3 bytes, contiguous in HBM).
 // Four workgroups on the same XCD (a "quad") walk the same tile sequence, one workgroup per compute unit,
 // 4 wavefronts each (one per SIMD, 512 registers).  Member m of the quad owns
-//   * batch rows 32m..32m+31 for the logits and the sigmoid ("stage A"), and
+//   * label rows 16m..16m+15 of every tile for the logits and the sigmoid ("stage A"), and
 //   * input features 192m..192m+191 for grad_X, grad_W and the in-place update ("stage B"),
-// so no arithmetic is repeated and every weight byte is read from HBM once and written once per step.
-// The only data the members exchange is G = sigmoid(logits) - target in bf16 (4.5 KiB per member and tile),
-// through a small ring of slots in global memory that stays in the XCD's L2, guarded by per-member
-// "tiles published" counters.  Stage A runs three tiles ahead of stage B, so neither the exchange nor the
+// so no arithmetic is repeated and every weight byte is read from HBM once and written once per step.  A member
+// reads 24 KiB per tile (its rows and its columns), always as whole 16-byte pieces of contiguous row segments
+// sent straight to LDS: the vector memory path of a compute unit handles few cache lines per clock, and
+// register loads in MFMA operand order (16 rows x 64 bytes per instruction) would keep it busy longer than
+// the MFMAs run.
+// The only data the members exchange is G = sigmoid(logits) - target in bf16 (4 KiB per member and tile),
+// through a small ring of slots in global memory, guarded by per-member "tiles published" counters.  Stage A runs three tiles ahead of stage B, so neither the exchange nor the
 // counters are on the critical path.  Neither logits nor gradients ever reach HBM; the X operands of all three
 // GEMMs and the grad_X accumulators (96 KiB per compute unit) live in registers for the whole launch.
 //
-//   stage A(t): Z[64 x 32] = W_t Xq_m^T        v_mfma_f32_16x16x128_f8f6f4; wavefront w takes rows 16w..16w+15,
-//                                              its W rows come straight from L2 into registers
+//   stage A(t): Z[16 x 128] = W_t[16m.., :] Xq^T  v_mfma_f32_16x16x128_f8f6f4; wavefront w takes batch rows 32w..32w+31,
+//                                              the 16 W rows are read from LDS by all four wavefronts
 //               G = bf16(sigmoid(bf16(Z))) - [positive], stored to the exchange slot in [b][l] order
-//   stage B(t): the four G parts arrive in LDS by global_load_lds; wavefront w takes features 48w..48w+47
+//   stage B(t): the whole G tile arrives in LDS by global_load_lds; wavefront w takes features 48w..48w+47
 //               grad_X[128 x 48] += G^T W_t      v_mfma_f32_16x16x32_bf16, W via ds_read_b64_tr_b8 + fp8->bf16
 //               A^T[48 x 64]     = X^T G^T        v_mfma_f32_16x16x32_bf16, G via ds_read_b64_tr_b16
 //               W_t              = round(W - lr A) from registers to memory, 12 bytes per lane
@@ -34,14 +37,18 @@ constexpr int QCOLS = D / 4;              // features owned by one member (192)
 constexpr int QWS = QCOLS + 16;           // LDS row stride of the own-column tile image (13 x 16 bytes)
 constexpr int QWC_BYTES = TL * QWS;       // 13312
 constexpr int QRING = 6;                  // own-column tile images in flight
-constexpr int QPL_S = TL * 2 + 16;        // bytes per batch row of a G plane ([32 b][64 l] bf16 + pad)
-constexpr int QPLANE = 5120;              // bytes per plane (32 x 144 = 4608, padded to 5 KiB)
-constexpr int QG_BYTES = 4 * QPLANE;      // one gathered G tile
+constexpr int QPL_S = TL * 2 + 16;        // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
+constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432), padded to 20 wave-wide loads
 constexpr int QSLOTS = 8;                 // exchange slots per quad
 constexpr int QLDS_G = QRING * QWC_BYTES; // LDS offset of the two gathered-G buffers
-constexpr int QLDS_BYTES = QLDS_G + 2 * QG_BYTES;
+constexpr int QRS = D + 16;               // LDS row stride of the own-rows image (49 x 16 bytes)
+constexpr int QROW_BYTES = 13 * 1024;     // 16 rows x 784 = 12544, padded to 13 wave-wide loads
+constexpr int QRRING = 3;                 // own-rows images in flight
+constexpr int QLDS_R = QLDS_G + 2 * QG_BYTES;
+constexpr int QLDS_BYTES = QLDS_R + QRRING * QROW_BYTES;
 constexpr int QSPIN_LIMIT = 1 << 18;
-constexpr int QAHEAD = 3;                 // stage A runs this many tiles ahead of stage B
+constexpr int QAHEAD = 4;                 // stage A runs this many tiles ahead of stage B
+constexpr int QINF = QAHEAD + 3;          // tile descriptors held in scalar registers
 
 struct QuadParams {
   unsigned char* chunk[MAX_CHUNKS];   // device pointers of the chunk weight tensors [rows_per_chunk, 768] e4m3
@@ -54,8 +61,9 @@ struct QuadParams {
   const bf16x8* xt;                   // grad_W operands
   const unsigned* keys;               // sorted positives: label*256 + batch_row
   const int* tile_ptr;                // [num_tiles+1] offsets into keys
+  const uint4* desc;                  // [num_tiles][2] tile descriptors written by tile_desc_kernel
   floatx4* partial;                   // [gridDim.x][24][256] per-workgroup grad_X partial sums
-  unsigned char* exch;                // [nquads][QSLOTS][4][QPLANE] G exchange ring
+  unsigned char* exch;                // [nquads][QSLOTS][QG_BYTES] G exchange ring
   int* flags;                         // [nquads][4] tiles-published counters; [nquads*4] error word; then xcc ids
   float zscale;                       // scale_w * scale_x applied to the logits accumulator
   float lr_eff;                       // lr / scale_w
@@ -64,6 +72,13 @@ struct QuadParams {
 
 #ifndef XMC_DBG_SKIP
 #define XMC_DBG_SKIP 0   // timing experiments only: bit mask of phases to leave out (results are then wrong)
+#endif
+#ifdef XMC_TIMING   // timing experiments only: per-wavefront clock totals of the phases of the main loop
+#define QT_DECL unsigned long long tprev = __builtin_amdgcn_s_memtime(); unsigned tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define QT(k) { __builtin_amdgcn_sched_barrier(0); unsigned long long tn = __builtin_amdgcn_s_memtime(); tacc[k] += (unsigned)(tn - tprev); tprev = tn; __builtin_amdgcn_sched_barrier(0); }
+#else
+#define QT_DECL
+#define QT(k)
 #endif
 #define QFENCE() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point
 typedef __attribute__((address_space(3))) unsigned char qlds_u8;
@@ -93,23 +108,35 @@ __device__ __forceinline__ bf16x8 q_fp8x8_to_bf16x8(intx2 raw) {
                 (__bf16)f45.x, (__bf16)f45.y, (__bf16)f67.x, (__bf16)f67.y};
 }
 
-// Everything the kernel needs to know about one tile; wave-uniform, kept in scalar registers and computed
-// several iterations before it is used so that the scalar-memory latency stays off the critical path.
-struct QTile { unsigned char* base; int c, row0, rows_valid, p0, p1; unsigned seed; };
+// Everything the kernel needs to know about one tile; wave-uniform, kept in scalar registers.  The descriptors are
+// precomputed by tile_desc_kernel and fetched with ordinary vector loads several iterations ahead, so that they
+// travel in the same in-order queue as the other prefetches and never stall the wavefront the way a scalar load
+// followed by an LDS wait would.
+struct QTile { unsigned char* base; unsigned label0; int row0, rows_valid, p0, p1; unsigned seed; };
 
-__device__ __forceinline__ QTile q_tile(const QuadParams& p, int t) {
+__device__ __forceinline__ QTile q_from_desc(uint4 d0, uint4 d1) {
   QTile q;
-  const __attribute__((address_space(4))) int* ctile_ptr = (const __attribute__((address_space(4))) int*)p.tile_ptr;
-  const bool valid = t < p.num_tiles;
-  const int tt = valid ? t : 0;
-  q.c = tt / p.tiles_per_chunk;
-  q.row0 = (tt - q.c * p.tiles_per_chunk) * TL;
-  q.rows_valid = min(TL, p.rows_per_chunk - q.row0);
-  q.base = p.chunk[q.c] + (size_t)q.row0 * D;
-  q.seed = p.seed[q.c];
-  q.p0 = ctile_ptr[tt];
-  q.p1 = valid ? ctile_ptr[tt + 1] : q.p0;
+  const unsigned lo = __builtin_amdgcn_readfirstlane(d0.x), hi = __builtin_amdgcn_readfirstlane(d0.y);
+  q.base = (unsigned char*)(((unsigned long long)hi << 32) | lo);
+  q.seed = __builtin_amdgcn_readfirstlane(d0.z);
+  q.p0 = (int)__builtin_amdgcn_readfirstlane(d0.w);
+  q.p1 = (int)__builtin_amdgcn_readfirstlane(d1.x);
+  q.row0 = (int)__builtin_amdgcn_readfirstlane(d1.y);
+  q.rows_valid = (int)__builtin_amdgcn_readfirstlane(d1.z);
+  q.label0 = __builtin_amdgcn_readfirstlane(d1.w);
   return q;
+}
+
+// desc[t] = {base pointer, seed, first key, one past last key | row in chunk, valid rows, first label, -}
+__global__ void tile_desc_kernel(const QuadParams p, uint4* desc) {
+  int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= p.num_tiles) return;
+  const int c = t / p.tiles_per_chunk;
+  const int row0 = (t - c * p.tiles_per_chunk) * TL;
+  const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
+  desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), p.seed[c], (unsigned)p.tile_ptr[t]};
+  desc[2 * t + 1] = uint4{(unsigned)p.tile_ptr[t + 1], (unsigned)row0, (unsigned)min(TL, p.rows_per_chunk - row0),
+                          (unsigned)(c * p.rows_per_chunk + row0)};
 }
 
 template <int MODE>
@@ -132,12 +159,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   if (tid == 0) p.flags[nquads * 4 + 1 + g] = (int)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15);   // XCC_ID
 
   // ---- resident operands
-  intx8 xq[2][6];      // logits: batch blocks 32m + 16nb.., K steps of 128
+  intx8 xq[2][6];      // logits: batch blocks 32w + 16nb.., K steps of 128
 #pragma unroll
   for (int nb = 0; nb < 2; nb++)
 #pragma unroll
     for (int ks = 0; ks < 6; ks++)
-      xq[nb][ks] = *(const intx8*)(p.xq + ((size_t)(((m * 2 + nb) * 6 + ks) * 64 + lane)) * 32);
+      xq[nb][ks] = *(const intx8*)(p.xq + ((size_t)(((w * 2 + nb) * 6 + ks) * 64 + lane)) * 32);
   bf16x8 xt[3][4];     // grad_W: feature blocks of this wavefront's 48 features, K steps of 32 batch rows
 #pragma unroll
   for (int cg = 0; cg < 3; cg++)
@@ -149,46 +176,61 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 #pragma unroll
     for (int b = 0; b < 3; b++) acc2[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  QT_DECL
   // own-column tile image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 wave-wide loads; every
   // wavefront issues exactly four (three of the sixteen are harmless repeats)
-  auto issue_wcol = [&](int i, const QTile& q) {
+  auto wcol_piece = [&](int i, const QTile& q, int s) {
     if (i >= n_it || (XMC_DBG_SKIP & 32)) return;
     const unsigned dst = (unsigned)((i % QRING) * QWC_BYTES);
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      int piece = (w + 4 * s) % 13;
-      int ch = piece * 64 + lane;
-      int row = ch / 13, cc = ch - row * 13;
-      row = min(row, q.rows_valid - 1);
-      cc = min(cc, 11);
-      q_lds_load16(q.base + (size_t)row * D + QCOLS * m + cc * 16, dst + piece * 1024);
-    }
+    int piece = (w + 4 * s) % 13;
+    int ch = piece * 64 + lane;
+    int row = ch / 13, cc = ch - row * 13;
+    row = min(row, q.rows_valid - 1);
+    cc = min(cc, 11);
+    q_lds_load16(q.base + (size_t)row * D + QCOLS * m + cc * 16, dst + piece * 1024);
   };
-  // rows 16w..16w+15 of tile i as logits operands: lane (row l16, k group kg) holds 32 consecutive bytes per K step
-  auto load_a = [&](int i, const QTile& q, uint4 (&a)[12]) {
+  auto issue_wcol = [&](int i, const QTile& q) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) wcol_piece(i, q, s);
+  };
+  // own-rows image: rows 16m..16m+15 of tile i, 16 x 49 chunks of 16 bytes (48 data + 1 pad) = 13 wave-wide loads
+  auto rows_piece = [&](int i, const QTile& q, int s) {
     if (i >= n_it || (XMC_DBG_SKIP & 512)) return;
-    const unsigned char* src = q.base + (size_t)min(16 * w + l16, q.rows_valid - 1) * D + kg * 32;
-#pragma unroll
-    for (int ks = 0; ks < 6; ks++) {
-      a[2 * ks] = *(const uint4*)(src + ks * 128);
-      a[2 * ks + 1] = *(const uint4*)(src + ks * 128 + 16);
-    }
+    const unsigned dst = (unsigned)(QLDS_R + (i % QRRING) * QROW_BYTES);
+    int piece = (w + 4 * s) % 13;
+    int ch = piece * 64 + lane;
+    int row = ch / 49, cc = ch - row * 49;
+    row = max(min(16 * m + min(row, 15), q.rows_valid - 1), 0);
+    cc = min(cc, 47);
+    q_lds_load16(q.base + (size_t)row * D + cc * 16, dst + piece * 1024);
   };
-  // stage A of tile i: logits, sigmoid minus target, store this member's G part to the exchange slot
-  // (published later, once the stores have completed)
-  auto stage_a = [&](int i, const QTile& q, const uint4 (&a)[12]) {
+  auto issue_rows = [&](int i, const QTile& q) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) rows_piece(i, q, s);
+  };
+  // stage A of tile i: logits of label rows 16m.. against batch rows 32w.., sigmoid minus target, store this
+  // wavefront's part of G to the exchange slot (published later, once the stores have completed)
+  auto stage_a = [&](int i, const QTile& q) {
     if (i >= n_it) return;
     floatx4 z[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-    if (!(XMC_DBG_SKIP & 1))
+    if (!(XMC_DBG_SKIP & 1)) {
+      // lane (row l16, k group kg) holds 32 consecutive bytes per K step
+      const unsigned asrc = (unsigned)(QLDS_R + (i % QRRING) * QROW_BYTES) + l16 * QRS + kg * 32;
+      intx4 alo[6], ahi[6];
 #pragma unroll
-    for (int ks = 0; ks < 6; ks++) {
-      intx8 av = intx8{(int)a[2 * ks].x, (int)a[2 * ks].y, (int)a[2 * ks].z, (int)a[2 * ks].w,
-                       (int)a[2 * ks + 1].x, (int)a[2 * ks + 1].y, (int)a[2 * ks + 1].z, (int)a[2 * ks + 1].w};
-      z[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, xq[0][ks], z[0], 0, 0, 0, 0, 0, 0);
-      z[1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, xq[1][ks], z[1], 0, 0, 0, 0, 0, 0);
+      for (int ks = 0; ks < 6; ks++) {
+        alo[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128);
+        ahi[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128 + 16);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 6; ks++) {
+        intx8 av = intx8{alo[ks].x, alo[ks].y, alo[ks].z, alo[ks].w, ahi[ks].x, ahi[ks].y, ahi[ks].z, ahi[ks].w};
+        z[0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, xq[0][ks], z[0], 0, 0, 0, 0, 0, 0);
+        z[1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, xq[1][ks], z[1], 0, 0, 0, 0, 0, 0);
+      }
     }
     const float nlog2e = -1.44269504088896340736f;
-    const int r0 = 16 * w + 4 * kg;
+    const int r0 = 16 * m + 4 * kg;   // this lane's label rows r0..r0+3; its batch rows are 32w + 16nb + l16
     float sg[2][4];
 #pragma unroll
     for (int nb = 0; nb < 2; nb++)
@@ -200,12 +242,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       }
     // positives of this tile (set semantics: a repeated key counts once); wave-uniform scalar loads
     if (q.p1 > q.p0) {
-      const unsigned label0 = (unsigned)(q.c * p.rows_per_chunk + q.row0);
+      const unsigned label0 = q.label0;
       for (int e = q.p0; e < q.p1; e++) {
         const unsigned key = ckeys[e];
         const unsigned prev = e > 0 ? ckeys[e - 1] : ~key;
         const unsigned l = (key >> 8) - label0 - (unsigned)r0;
-        const unsigned bl = (key & 255u) - (unsigned)(32 * m) - (unsigned)l16;     // 0 or 16 for this lane's blocks
+        const unsigned bl = (key & 255u) - (unsigned)(32 * w) - (unsigned)l16;     // 0 or 16 for this lane's blocks
         if (prev != key && l < 4u && (bl == 0u || bl == 16u)) {
 #pragma unroll
           for (int nb = 0; nb < 2; nb++)
@@ -215,7 +257,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         }
       }
     }
-    unsigned char* plane = p.exch + ((size_t)((quad * QSLOTS + (i & (QSLOTS - 1))) * 4 + m)) * QPLANE;
+    unsigned char* plane = p.exch + ((size_t)(quad * QSLOTS + (i & (QSLOTS - 1)))) * QG_BYTES + 32 * w * QPL_S;
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
       unsigned short sb[4];
@@ -227,42 +269,66 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       *(uint2*)(plane + (16 * nb + l16) * QPL_S + r0 * 2) = v;
     }
   };
-  // wait until every member has published at least `need` tiles (f: an earlier reading of the counters)
+  // wait until every member has published at least `need` tiles (f: an earlier reading of the counters, which
+  // normally suffices; the polling loop is kept out of the common path so that it costs no memory wait)
   auto wait_published = [&](int need, int f) {
     if (XMC_DBG_SKIP & 128) return;
+    if (__builtin_amdgcn_read_exec() == __builtin_amdgcn_ballot_w64(f >= need)) return;
     for (int spin = 0;; spin++) {
-      int ok = f >= need;
-      if (__builtin_amdgcn_read_exec() == __builtin_amdgcn_ballot_w64(ok)) break;
+      f = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (__builtin_amdgcn_read_exec() == __builtin_amdgcn_ballot_w64(f >= need)) break;
       if (spin >= QSPIN_LIMIT || ((spin & 1023) == 1023 && __hip_atomic_load(errw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
         if (lane == 0) __hip_atomic_store(errw, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
       __builtin_amdgcn_s_sleep(2);
-      f = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   };
-  // gather the four G parts of tile i: 20 wave-wide loads of 1 KiB, five per wavefront
-  auto issue_gather = [&](int i) {
+  // gather the G tile of tile i: 20 wave-wide loads of 1 KiB, five per wavefront
+  auto gather_piece = [&](int i, int s) {
     if (i >= n_it || (XMC_DBG_SKIP & 256)) return;
-    const unsigned char* src = p.exch + ((size_t)((quad * QSLOTS + (i & (QSLOTS - 1))) * 4)) * QPLANE;
+    const unsigned char* src = p.exch + ((size_t)(quad * QSLOTS + (i & (QSLOTS - 1)))) * QG_BYTES;
     const unsigned dst = (unsigned)(QLDS_G + (i & 1) * QG_BYTES);
+    int piece = w + 4 * s;
+    // The slot was written by other compute units of this XCD and is read from the shared L2.  This compute unit's
+    // own L1 may still hold the slot's previous contents, so the L1 (and only the L1) is invalidated first; nothing
+    // else this kernel loads is ever reused from it.
+    if (s == 0) asm volatile("buffer_inv sc0" ::: "memory");
+    q_lds_load16(src + piece * 1024 + lane * 16, dst + piece * 1024);
+  };
+  auto issue_gather = [&](int i) {
 #pragma unroll
-    for (int s = 0; s < 5; s++) {
-      int piece = w + 4 * s;
-      q_lds_load16_l2(src + piece * 1024 + lane * 16, dst + piece * 1024);
-    }
+    for (int s = 0; s < 5; s++) gather_piece(i, s);
   };
 
-  // ---- prologue: own columns of tiles 0..4 in flight, stage A of tiles 0..2, gather of tile 0, rows of tile 3
-  uint4 areg[12];
-  QTile inf[6];        // inf[k] describes the tile k positions ahead of the current one
+  // ---- prologue: own columns of tiles 0..4 in flight, stage A of the first QAHEAD tiles, own rows of the next two,
+  //      gather of tile 0
+  auto load_desc = [&](int i, uint4& d0, uint4& d1) {
+    const int t = quad + nquads * i;
+    const uint4* src = p.desc + 2 * (size_t)(t < p.num_tiles ? t : 0);
+    d0 = src[0];
+    d1 = src[1];
+  };
+  QTile inf[QINF];     // inf[k] describes the tile k positions ahead of the current one
 #pragma unroll
-  for (int k = 0; k < 6; k++) inf[k] = q_tile(p, quad + nquads * k);
+  for (int k = 0; k < QINF; k++) {
+    uint4 d0, d1;
+    load_desc(k, d0, d1);
+    inf[k] = q_from_desc(d0, d1);
+  }
+#pragma unroll
+  for (int k = 0; k < 3; k++) issue_rows(k, inf[k]);
 #pragma unroll
   for (int k = 0; k < 5; k++) issue_wcol(k, inf[k]);
 #pragma unroll
-  for (int k = 0; k < QAHEAD; k++) { load_a(k, inf[k], areg); stage_a(k, inf[k], areg); }
-  load_a(QAHEAD, inf[QAHEAD], areg);
+  for (int k = 0; k < QAHEAD; k++) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    stage_a(k, inf[k]);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (k + 3 < QAHEAD + 2) issue_rows(k + 3, inf[k + 3]);
+  }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0 && n_it > 0) __hip_atomic_store(flags + m, min(QAHEAD, n_it), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -270,23 +336,40 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   issue_gather(0);
   int fseen = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
+  bool prev_full = false;
   for (int i = 0; i < n_it; i++) {
     const QTile q = inf[0];
     const unsigned wc = (unsigned)((i % QRING) * QWC_BYTES);
     const unsigned gb = (unsigned)(QLDS_G + (i & 1) * QG_BYTES);
-    // tile six positions ahead: its scalar loads complete under the wait below
-    const QTile qnew = q_tile(p, quad + nquads * (i + 6));
-
-    // everything issued during the previous iteration has landed: G of tile i, own columns up to tile i+4, this
-    // member's G part of tile i+2, the rows of tile i+3
-    __builtin_amdgcn_s_waitcnt(0);
+    uint4 dnext0, dnext1;   // descriptor of the tile QINF positions ahead, fetched below
+    // Vector memory operations retire in order.  The last four this wavefront issued in the previous iteration are
+    // the stores of updated weights; everything older - G of tile i, own columns and own rows of the tiles ahead,
+    // this member's G part of tile i+QAHEAD-1, the counters - was issued half an iteration earlier or more.
+    // Leaving four operations in flight keeps the store latency off the critical path.  If the
+    // previous tile was not full, fewer stores were issued and the count could cover loads, so all are waited for.
+    if (prev_full) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    QT(0)
     __syncthreads();
+    prev_full = q.rows_valid == TL;
     if (tid == 0 && i > 0 && i + QAHEAD - 1 < n_it)
       __hip_atomic_store(flags + m, i + QAHEAD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    QT(1)
 
-    stage_a(i + QAHEAD, inf[QAHEAD], areg);
-    load_a(i + QAHEAD + 1, inf[QAHEAD + 1], areg);
-    issue_wcol(i + 5, inf[5]);
+    stage_a(i + QAHEAD, inf[QAHEAD]);
+    QT(2)
+    // G of the next tile was published by every member at least one full iteration ago, so the counters read at the
+    // end of the previous iteration normally suffice
+    if (i + 1 < n_it) wait_published(i + 2, fseen);
+    // the 13 direct-to-LDS loads of this iteration (G of tile i+1, own rows of tile i+5, own columns of tile i+5),
+    // issued one by one between the MFMAs below so that the memory pipeline never makes the wavefront wait
+    auto mem_piece = [&](int k) {
+      if (k < 5) gather_piece(i + 1, k);
+      else if (k < 9) rows_piece(i + QAHEAD + 2, inf[QAHEAD + 2], k - 5);
+      else if (k < 13) wcol_piece(i + 5, inf[5], k - 9);
+      else load_desc(i + QINF, dnext0, dnext1);
+    };
+    QT(3)
 
     // ---- grad_X[128 x 48] += G^T W; 6 steps (32-row K step major, 16-feature block minor); the transposed W read
     //      of step s+2 and the fp8->bf16 conversion of step s+1 are issued between the MFMAs of step s
@@ -295,7 +378,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       const unsigned gsrc = gb + l16 * QPL_S + kg * 16;
       bf16x8 ga[2][8];
 #pragma unroll
-      for (int mb = 0; mb < 8; mb++) ga[0][mb] = *(const bf16x8*)(lds + gsrc + (mb >> 1) * QPLANE + 16 * (mb & 1) * QPL_S);
+      for (int mb = 0; mb < 8; mb++) ga[0][mb] = *(const bf16x8*)(lds + gsrc + 16 * mb * QPL_S);
       intx2 raw[3];
       raw[0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(lds + wsrc));
       raw[1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(lds + wsrc + 16));
@@ -311,7 +394,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 #pragma unroll
           for (int u = 0; u < 4; u++) {
             const int mb = 4 * s + u;
-            ga[1][mb] = *(const bf16x8*)(lds + gsrc + (mb >> 1) * QPLANE + 16 * (mb & 1) * QPL_S + 64);
+            ga[1][mb] = *(const bf16x8*)(lds + gsrc + 16 * mb * QPL_S + 64);
           }
         }
         QFENCE();
@@ -320,23 +403,33 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
           acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[ks2][mb], wb[s & 1], acc2[mb][nn], 0, 0, 0);
           if (mb == 1 && s + 1 < 6) wb[(s + 1) & 1] = q_fp8x8_to_bf16x8(raw[(s + 1) % 3]);
           if (mb == 1) QFENCE();
+          if (mb == 3) { mem_piece(2 * s); QFENCE(); }
+          if (mb == 6) { mem_piece(2 * s + 1); QFENCE(); }
+          if (mb == 7 && s == 4) { mem_piece(12); QFENCE(); }
+          if (mb == 7 && s == 5) { mem_piece(13); QFENCE(); }
         }
         QFENCE();
       }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 14; k++) mem_piece(k);
     }
 
+    QT(4)
+    // the counters, read before this iteration's stores so that the wait at the top of the loop covers the load
+    fseen = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- A^T[48 features x 64 rows] = X^T G^T in four 16-row blocks; the update of block nb-1 (VALU, registers to
     //      memory) is issued between the MFMAs of block nb.  Row r = 4kg+e of feature block cg is feature
     //      12kg + 4cg + e of the wavefront's 48, so that a lane ends up with 12 consecutive bytes of one weight row.
     {
       const unsigned bsrc = gb + (8 * kg + (l16 >> 2)) * QPL_S + 4 * (l16 & 3) * 2;
       const unsigned wrow = wc + l16 * QWS + 48 * w + 12 * kg;
-      const unsigned grow0 = (unsigned)(q.c * p.rows_per_chunk + q.row0 + l16);
+      const unsigned grow0 = q.label0 + (unsigned)l16;
       auto load_bg = [&](int nb, bf16x8 (&bg)[4]) {
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-          shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4*)(lds + bsrc + ks * QPLANE + 16 * nb * 2));
-          shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4*)(lds + bsrc + ks * QPLANE + 16 * nb * 2 + 4 * QPL_S));
+          shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4*)(lds + bsrc + ks * 32 * QPL_S + 16 * nb * 2));
+          shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4*)(lds + bsrc + ks * 32 * QPL_S + 16 * nb * 2 + 4 * QPL_S));
           bg[ks] = __builtin_bit_cast(bf16x8, shortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
         }
       };
@@ -383,18 +476,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       }
     }
 
-    // ---- G of the next tile: published by every member at least one full iteration ago, so the counters read at
-    //      the end of the previous iteration normally suffice
-    if (i + 1 < n_it) {
-      wait_published(i + 2, fseen);
-      issue_gather(i + 1);
-    }
-    fseen = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    QT(5)
+    QT(6)
 #pragma unroll
-    for (int k = 0; k < 5; k++) inf[k] = inf[k + 1];
-    inf[5] = qnew;
+    for (int k = 0; k + 1 < QINF; k++) inf[k] = inf[k + 1];
+    inf[QINF - 1] = q_from_desc(dnext0, dnext1);
   }
 
+#ifdef XMC_TIMING
+  if (lane == 0 && g < 96)
+    for (int k = 0; k < 8; k++) p.flags[1024 + (g * 4 + w) * 8 + k] = (int)tacc[k];
+#endif
   // ---- per-workgroup grad_X partial, summed in a fixed order by reduce_gx_quad_kernel
   floatx4* dst = p.partial + (size_t)g * 24 * QNT;
 #pragma unroll

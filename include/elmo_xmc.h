@@ -79,6 +79,10 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
  * then forgets them.  Pass nulls to cancel. */
 int xmc_profile_events(void* start_event, void* stop_event);
 
+/* Measurement aid (no counterpart in the reference): copies `bytes` (a multiple of 16) from src to dst with a plain
+ * grid-stride kernel.  Memory-traffic counters are calibrated against this launch of known size. */
+int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
+
 /* Reads back the error word a step leaves in the workspace (non-zero: a workgroup gave up waiting for its
  * partner).  Synchronises the stream; meant for tests and debugging, not for the training loop. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
