@@ -182,7 +182,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
-    reduce_gx_quad_kernel<<<96, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+    reduce_gx_quad_kernel<<<48, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
                                                  (unsigned short*)grad_x_bf16, batch);
   }
   return launch_status();
