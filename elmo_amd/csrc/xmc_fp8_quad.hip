@@ -439,7 +439,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
                                   (unsigned)(QCOLS * m + 48 * fg + 12 * kg + 4 * cg), q.seed);
         }
         if (row < q.rows_valid) {
-          unsigned* gp = (unsigned*)(q.base + (size_t)row * D + QCOLS * m + 48 * fg + 12 * kg);
+          // the pointer comes out of scalar registers as an integer: say that it is global memory, or the store
+          // becomes a flat one, which also counts as an LDS operation
+          typedef __attribute__((address_space(1))) unsigned gu32;
+          gu32* gp = (gu32*)(unsigned long long)(q.base + (size_t)row * D + QCOLS * m + 48 * fg + 12 * kg);
           gp[0] = outw[0]; gp[1] = outw[1]; gp[2] = outw[2];
         }
       }
