@@ -177,7 +177,8 @@ def main():
                    "lr": cfg.lr, "rounding": args.round, "seed": cfg.seed},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "fp8_step_kernel", "kernel_ms": kernel_ms,
+                     "kernel": "fp8_step_kernel" if os.environ.get("XMC_KERNEL") == "pair" else "fp8_step_quad_kernel",
+                     "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_flops_per_launch": algo_flops},
         "roofline_step_frac": t_roof / (ms_per_step * 1e-3),
         "roofline_steps_per_s": 1.0 / t_roof,

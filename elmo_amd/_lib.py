@@ -37,6 +37,8 @@ def load():
     lib.xmc_fp8_forward.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp, sz, vp]
     lib.xmc_step_error_word.restype = i32
     lib.xmc_step_error_word.argtypes = [vp, i32, i32, vp]
+    lib.xmc_select_step_kernel.restype = i32
+    lib.xmc_select_step_kernel.argtypes = [i32]
     lib.xmc_copy_probe.restype = i32
     lib.xmc_copy_probe.argtypes = [vp, vp, sz, vp]
     lib.xmc_profile_events.restype = i32

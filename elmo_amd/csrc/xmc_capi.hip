@@ -59,6 +59,16 @@ __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
 
+// which fused kernel xmc_fp8_step launches: 0 = quad (default), 1 = pair; initial value from XMC_KERNEL=pair|quad
+int g_step_kernel = -1;
+int step_kernel_choice() {
+  if (g_step_kernel < 0) {
+    const char* e = getenv("XMC_KERNEL");
+    g_step_kernel = (e && !__builtin_strcmp(e, "pair")) ? 1 : 0;
+  }
+  return g_step_kernel;
+}
+
 int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
 
 }  // namespace
@@ -115,8 +125,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
                                                                 tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
-  static const bool use_pair = !(getenv("XMC_KERNEL") && !__builtin_strcmp(getenv("XMC_KERNEL"), "quad"));
-  if (use_pair) {
+  if (step_kernel_choice() == 1) {
     prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                                 (unsigned short*)(ws + WS_XT));
     StepParams p;
@@ -217,6 +226,12 @@ int xmc_profile_events(void* start_event, void* stop_event) {
   return XMC_OK;
 }
 
+int xmc_select_step_kernel(int which) {
+  if (which < 0 || which > 1) return XMC_ERR_MODE;
+  g_step_kernel = which;
+  return XMC_OK;
+}
+
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream_) {
   if (!dst || !src) return XMC_ERR_NULL;
   if (!aligned16(dst) || !aligned16(src) || bytes % 16 != 0) return XMC_ERR_ALIGN;
@@ -230,7 +245,8 @@ int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chun
   if (!workspace) return XMC_ERR_NULL;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;
-  const int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;
+  int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;
+  if (step_kernel_choice() == 0) grid = grid / 32 * 32;   // the quad kernel keeps the word behind its counters
   int word = 0;
   if (hipMemcpyAsync(&word, (const unsigned char*)workspace + WS_FLAGS + (size_t)grid * 4, 4, hipMemcpyDeviceToHost,
                      (hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;

@@ -79,6 +79,12 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
  * then forgets them.  Pass nulls to cancel. */
 int xmc_profile_events(void* start_event, void* stop_event);
 
+/* Selects the fused kernel that xmc_fp8_step launches (no counterpart in the reference): 0 = four compute units per
+ * tile stream without repeated arithmetic (default), 1 = two compute units per tile stream with the logits computed
+ * twice.  Both produce the same weights; grad_X differs by fp32 summation order only.  The environment variable
+ * XMC_KERNEL=pair|quad sets the initial choice. */
+int xmc_select_step_kernel(int which);
+
 /* Measurement aid (no counterpart in the reference): copies `bytes` (a multiple of 16) from src to dst with a plain
  * grid-stride kernel.  Memory-traffic counters are calibrated against this launch of known size. */
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);

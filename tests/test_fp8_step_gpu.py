@@ -60,6 +60,18 @@ def test_rtn_parity_small(gpu, nc, rows, batch, seed):
     check_rtn(case, gpu)
 
 
+@pytest.mark.parametrize("nc,rows,batch,seed", [(3, 208, 32, 13), (5, 2000, 64, 15), (2, 4096, 128, 14)])
+def test_rtn_parity_pair_kernel(gpu, nc, rows, batch, seed):
+    """The alternative fused kernel (two compute units per tile stream) meets the same bar."""
+    from elmo_amd import _lib
+    lib = _lib.load()
+    _lib.check(lib.xmc_select_step_kernel(1), "xmc_select_step_kernel")
+    try:
+        check_rtn(H.make_case(nc, rows, batch, seed), gpu)
+    finally:
+        _lib.check(lib.xmc_select_step_kernel(0), "xmc_select_step_kernel")
+
+
 def test_rtn_parity_medium_full_batch(gpu):
     case = H.make_case(2, 20000 // 16 * 16, 128, 21, pos_mean=5.4)
     frac = check_rtn(case, gpu)
