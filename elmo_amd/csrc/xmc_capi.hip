@@ -3,6 +3,7 @@
 #include "../../include/elmo_xmc.h"
 #include "xmc_fp8_step.hip"
 #include "xmc_fp8_quad.hip"
+#include "xmc_tiled.hip"
 #include <stdlib.h>
 
 using namespace xmc;
@@ -224,6 +225,85 @@ int xmc_profile_events(void* start_event, void* stop_event) {
   g_prof_start = (hipEvent_t)start_event;
   g_prof_stop = (hipEvent_t)stop_event;
   return XMC_OK;
+}
+
+size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk) {
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
+  const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
+  const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
+  return TW_G + 2 * rows_pad * BP * 2 + ((tiles + 1) * 4 + 255) / 256 * 256;
+}
+
+int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                   const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
+                   const uint32_t* seeds, int round_mode, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                   size_t workspace_bytes, void* stream_) {
+  if (!chunk_ptrs || !x_bf16 || !workspace || !grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
+  if (features != D || batch <= 0 || batch > BP) return XMC_ERR_SHAPE;
+  if (rows_per_chunk <= 0 || rows_last_chunk <= 0 || rows_last_chunk > rows_per_chunk) return XMC_ERR_SHAPE;
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
+  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1 || nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
+  if (weight_type != W_E4M3 && weight_type != W_BF16) return XMC_ERR_MODE;
+  if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX) return XMC_ERR_MODE;
+  if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
+  for (int c = 0; c < num_chunks; c++) {
+    if (!chunk_ptrs[c]) return XMC_ERR_NULL;
+    if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
+  }
+  if (!aligned16(x_bf16) || ((uintptr_t)workspace & 255) != 0) return XMC_ERR_ALIGN;
+  if (workspace_bytes < xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk)) return XMC_ERR_WORKSPACE;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  unsigned char* ws = (unsigned char*)workspace;
+
+  const int rows_pad = (rows_per_chunk + TL - 1) / TL * TL;
+  const int tiles_per_chunk = rows_pad / TL;
+  const int num_tiles = num_chunks * tiles_per_chunk;
+  unsigned short* xb = (unsigned short*)(ws + TW_XB);
+  unsigned short* xT = (unsigned short*)(ws + TW_XT);
+  unsigned* keys = (unsigned*)(ws + TW_KEYS);
+  float* gx_total = (float*)(ws + TW_GX);
+  floatx4* partial = (floatx4*)(ws + TW_PART);
+  unsigned short* glb = (unsigned short*)(ws + TW_G);
+  unsigned short* gbl = glb + (size_t)rows_pad * BP;
+  int* tile_ptr = (int*)(gbl + (size_t)rows_pad * BP);
+  int n_pad = 0;
+  if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
+
+  if (n_pad > 0)
+    sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys);
+  tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
+  tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, xb, xT);
+  tiled_zero_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>(gx_total, BP * D);
+  for (int c = 0; c < num_chunks; c++) {
+    void* w = chunk_ptrs[c];
+    const int rows = c == num_chunks - 1 ? rows_last_chunk : rows_per_chunk;
+    const int rp = (rows + TL - 1) / TL * TL;           // padded rows of this chunk (G buffers use the stride rows_pad)
+    const int tiles = rp / TL;
+    const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;
+    const unsigned seed = seeds ? seeds[c] : 0u;
+    int range = (rp + T_SPLITS - 1) / T_SPLITS;
+    range = (range + TL - 1) / TL * TL;
+    const int splits = (rp + range - 1) / range;
+    if (weight_type == W_BF16) {
+      tiled_logits_kernel<W_BF16><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tile_ptr + c * tiles_per_chunk, label0, glb, gbl);
+      tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
+    } else {
+      tiled_logits_kernel<W_E4M3><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tile_ptr + c * tiles_per_chunk, label0, glb, gbl);
+      tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
+    }
+    tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total);
+    if (weight_type == W_BF16) {
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+    } else {
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+    }
+  }
+  tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
+  return launch_status();
 }
 
 int xmc_select_step_kernel(int which) {

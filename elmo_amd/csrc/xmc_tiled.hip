@@ -1,0 +1,272 @@
+// Three-kernel ("tiled") classifier step for gfx950, for the two modes of the reference that keep bf16 temporaries:
+//   * bf16 weights          src/xmc_classifiers/chunked.py:85-131 with src/triton_kernels/stochastic_rounding_kernel.py:65-99
+//   * simulated FP8 weights src/xmc_classifiers/chunked_fp8xmc_clf.py:98-99,110,115-116 with
+//                           src/triton_kernels/fuse_kernel.py:134-199
+// Per chunk, as the reference does: logits -> G (sigmoid minus targets, bf16, kept in HBM in both orientations),
+// grad_X partial (split over label ranges, summed in a fixed order), grad_W + SGD update in place.  All three GEMMs
+// are bf16 v_mfma_f32_16x16x32_bf16 with fp32 accumulation; e4m3 weights are widened exactly on load.  These modes are
+// not the headline path: the kernels take their operands straight from global memory (L2) in MFMA operand order and
+// stage only the one operand that needs a transposition (W in grad_X) through LDS.
+#include "xmc_common.h"
+
+namespace xmc {
+
+enum WType { W_E4M3 = 0, W_BF16 = 1 };
+constexpr int T_SPLITS = 64;                       // label ranges of the grad_X kernel
+constexpr int T_WS2 = 48 * 2 + 16;                 // LDS row stride of a wavefront's W block, bytes
+
+typedef short tshortx4 __attribute__((ext_vector_type(4)));
+typedef short tshortx8 __attribute__((ext_vector_type(8)));
+
+// workspace of the tiled path (byte offsets, 256-byte aligned)
+constexpr size_t TW_XB = 0;                                        // X   [128][768] bf16, rows beyond the batch zero
+constexpr size_t TW_XT = TW_XB + (size_t)BP * D * 2;               // X^T [768][128] bf16
+constexpr size_t TW_KEYS = TW_XT + (size_t)BP * D * 2;             // sorted positive keys
+constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [128][768]
+constexpr size_t TW_PART = TW_GX + (size_t)BP * D * 4;             // grad_X partials [T_SPLITS][128*768] fp32
+constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // G [rows_pad][128] then G^T [128][rows_pad], then tile_ptr
+
+__device__ __forceinline__ bf16x8 t_fp8x8_to_bf16x8(intx2 raw) {
+  bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
+  bf16x2 c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.y, 1.0f, false), c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.y, 1.0f, true);
+  return bf16x8{c0.x, c0.y, c1.x, c1.y, c2.x, c2.y, c3.x, c3.y};
+}
+
+// eight consecutive weights of a row, starting at element index idx (a multiple of 8), as bf16
+template <int WT>
+__device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
+  if (WT == W_BF16) return *(const bf16x8*)((const unsigned short*)w + idx);
+  return t_fp8x8_to_bf16x8(*(const intx2*)((const unsigned char*)w + idx));
+}
+
+// X -> zero-padded row-major image and its transpose
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, unsigned short* xb, unsigned short* xT) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= BP * D) return;
+  int b = i / D, k = i - b * D;
+  unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
+  xb[i] = v;
+  xT[(size_t)k * BP + b] = v;
+}
+
+__global__ void tiled_zero_kernel(float* p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+// ---- logits, sigmoid minus targets.  One workgroup per 64 label rows, wavefront w takes rows 16w..16w+15 against the
+//      whole (padded) batch.  Writes G[l][b] and G^T[b][l]; rows beyond the chunk are written as zeros.
+template <int WT>
+__global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int rows, int rows_pad, const unsigned short* xb,
+                                                           const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
+                                                           unsigned short* glb, unsigned short* gbl) {
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int r0 = blockIdx.x * TL + 16 * wv;
+  const int lrow = min(r0 + l16, rows - 1);
+  floatx4 acc[8];
+#pragma unroll
+  for (int nb = 0; nb < 8; nb++) acc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int ks = 0; ks < D / 32; ks++) {
+    const bf16x8 a = t_load_w8<WT>(w, (size_t)lrow * D + 32 * ks + 8 * kg);
+#pragma unroll
+    for (int nb = 0; nb < 8; nb++) {
+      const bf16x8 b = *(const bf16x8*)(xb + (size_t)(16 * nb + l16) * D + 32 * ks + 8 * kg);
+      acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nb], 0, 0, 0);
+    }
+  }
+  // acc[nb][e] = Z[label r0 + 4kg + e][batch 16nb + l16]
+  const float nlog2e = -1.44269504088896340736f;
+  float sg[8][4];
+#pragma unroll
+  for (int nb = 0; nb < 8; nb++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float zf = bf16_rt(acc[nb][e]);
+      sg[nb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * nlog2e)));
+    }
+  // positives of this tile (set semantics: a repeated key counts once)
+  const int p0 = tile_ptr[blockIdx.x], p1 = tile_ptr[blockIdx.x + 1];
+  const unsigned lbase = label0_chunk + (unsigned)(r0 + 4 * kg);
+  for (int e = p0; e < p1; e++) {
+    const unsigned key = keys[e];
+    const unsigned prev = e > 0 ? keys[e - 1] : ~key;
+    const unsigned l = (key >> 8) - lbase;
+    const unsigned b = key & 255u;
+    if (prev != key && l < 4u && (b & 15u) == (unsigned)l16) {
+#pragma unroll
+      for (int nb = 0; nb < 8; nb++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++)
+          if ((b >> 4) == (unsigned)nb && l == (unsigned)q4) sg[nb][q4] = bf16_rt(sg[nb][q4] - 1.0f);
+    }
+  }
+#pragma unroll
+  for (int nb = 0; nb < 8; nb++) {
+    unsigned short sb[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[nb][e]) : (unsigned short)0;
+    const int b = 16 * nb + l16;
+    uint2 o;
+    o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
+    o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
+    *(uint2*)(gbl + (size_t)b * rows_pad + r0 + 4 * kg) = o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
+  }
+}
+
+// ---- grad_X partial of one label range: C[128 x 192] = G^T[128 x R] W[R x 192].  blockIdx = fb + 4*split; wavefront w
+//      owns features 192fb + 48w.. (3 blocks of 16) against all 8 batch blocks.  W goes through a wavefront-private LDS
+//      block and comes back transposed (ds_read_b64_tr_b16).
+template <int WT>
+__global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, const unsigned short* gbl,
+                                                          floatx4* partial) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[4 * 32 * T_WS2];
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int fb = blockIdx.x & 3, split = blockIdx.x >> 2;
+  const int f0 = 192 * fb + 48 * wv;
+  __attribute__((address_space(3))) unsigned char* lw = (__attribute__((address_space(3))) unsigned char*)lds_raw + wv * 32 * T_WS2;
+  floatx4 acc[8][3];
+#pragma unroll
+  for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+    for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int lbeg = split * range, lend = min(lbeg + range, bound);   // bound: this chunk's rows rounded up to a tile
+  for (int l0 = lbeg; l0 < lend; l0 += 32) {
+    // W[l0..l0+31][f0..f0+47] -> LDS as bf16, row stride T_WS2
+    if (WT == W_BF16) {
+#pragma unroll
+      for (int s = 0; s < 3; s++) {
+        const int c = lane + 64 * s, row = c / 6, c16 = c - row * 6;
+        const int lr = min(l0 + row, rows - 1);
+        const intx4 v = *(const intx4*)((const unsigned short*)w + (size_t)lr * D + f0 + 8 * c16);
+        *(__attribute__((address_space(3))) intx4*)(lw + row * T_WS2 + c16 * 16) = v;
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const int c = lane + 64 * s;
+        if (c < 96) {
+          const int row = c / 3, c16 = c - row * 3;
+          const int lr = min(l0 + row, rows - 1);
+          const intx4 v = *(const intx4*)((const unsigned char*)w + (size_t)lr * D + f0 + 16 * c16);
+          const bf16x8 lo = t_fp8x8_to_bf16x8(intx2{v.x, v.y}), hi = t_fp8x8_to_bf16x8(intx2{v.z, v.w});
+          *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32) = lo;
+          *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32 + 16) = hi;
+        }
+      }
+    }
+    bf16x8 ga[8];
+#pragma unroll
+    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gbl + (size_t)(16 * mb + l16) * rows_pad + l0 + 8 * kg);
+    bf16x8 wb[3];
+#pragma unroll
+    for (int nn = 0; nn < 3; nn++) {
+      const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * T_WS2 + (16 * nn + 4 * (l16 & 3)) * 2);
+      tshortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(lw + off));
+      tshortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(lw + off + 4 * T_WS2));
+      wb[nn] = __builtin_bit_cast(bf16x8, tshortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+    }
+#pragma unroll
+    for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+      for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
+  }
+  // acc[mb][nn][e] = C[batch 16mb + 4kg + e][feature f0 + 16nn + l16]
+  floatx4* dst = partial + ((size_t)split * 4 + fb) * 24 * 256;
+#pragma unroll
+  for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+    for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + tid] = acc[mb][nn];
+}
+
+// sum of the partials of one chunk in a fixed order; bf16 weights: the chunk's contribution is rounded to bf16 before it
+// is added to the fp32 total (chunked.py:116)
+__global__ __launch_bounds__(256) void tiled_reduce_kernel(const floatx4* partial, int splits, int round_bf16, float* gx_total) {
+  const int slot = blockIdx.x >> 2, fb = blockIdx.x & 3;
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < splits; sp++) s += partial[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
+  const int mb = slot / 3, nn = slot - mb * 3;
+  const int col = 192 * fb + 48 * wv + 16 * nn + l16;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int b = 16 * mb + 4 * kg + i;
+    const float v = round_bf16 ? bf16_rt(s[i]) : s[i];
+    gx_total[(size_t)b * D + col] += v;
+  }
+}
+
+__global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned short* gx_bf16, float* gx_f32) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= batch * D) return;
+  const float v = gx_total[i];
+  if (gx_f32) gx_f32[i] = v;
+  gx_bf16[i] = bf16_bits(v);
+}
+
+// ---- grad_W and the SGD update of one chunk, in place.  blockIdx = tile*4 + fb; wavefront w owns label rows 16w..16w+15
+//      of the tile and features 192fb.. (12 blocks of 16).  A^T[f][l] = sum_b X^T[f][b] G[l][b]; a lane ends up with four
+//      consecutive features of one label row.
+//        bf16 weights : a = bf16(A); t = w - lr*a; RTN: bf16(t);  SR: bits(t) + (philox(seed, l*768+f) & 0xFFFF), clear 16 bits
+//        e4m3 weights : t = w - lr*A;          RTN: e4m3(t) as torch casts (NaN above 464); SR: add 20 bits, clear, same cast
+template <int WT, int MODE>
+__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, const unsigned short* xT,
+                                                           float lr, unsigned seed) {
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int fb = blockIdx.x & 3, tile = blockIdx.x >> 2;
+  const int row = tile * TL + 16 * wv + l16;
+  bf16x8 gf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) gf[ks] = *(const bf16x8*)(glb + (size_t)row * BP + 32 * ks + 8 * kg);
+#pragma unroll 2
+  for (int nn = 0; nn < 12; nn++) {
+    const int f = 192 * fb + 16 * nn;
+    floatx4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      const bf16x8 xa = *(const bf16x8*)(xT + (size_t)(f + l16) * BP + 32 * ks + 8 * kg);
+      a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[ks], a, 0, 0, 0);
+    }
+    // a[e] = A[label row][feature f + 4kg + e]
+    if (row < rows) {
+      const int col = f + 4 * kg;
+      const size_t idx = (size_t)row * D + col;
+      float wv4[4];
+      if (WT == W_BF16) {
+        const uint2 raw = *(const uint2*)((const unsigned short*)w + idx);
+        wv4[0] = bf16_from_bits((unsigned short)(raw.x & 0xffffu)); wv4[1] = bf16_from_bits((unsigned short)(raw.x >> 16));
+        wv4[2] = bf16_from_bits((unsigned short)(raw.y & 0xffffu)); wv4[3] = bf16_from_bits((unsigned short)(raw.y >> 16));
+      } else {
+        const int raw = *(const int*)((const unsigned char*)w + idx);
+        floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, true);
+        wv4[0] = w01.x; wv4[1] = w01.y; wv4[2] = w23.x; wv4[3] = w23.y;
+      }
+      float t[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float g = WT == W_BF16 ? bf16_rt(a[e]) : a[e];
+        t[e] = __builtin_fmaf(-lr, g, wv4[e]);
+        if (MODE == ROUND_SR_PHILOX) {
+          const unsigned r = philox_word0((unsigned)row * (unsigned)D + (unsigned)(col + e), seed, 0u);
+          const unsigned mask = WT == W_BF16 ? 0xFFFFu : 0xFFFFFu;
+          t[e] = __uint_as_float((__float_as_uint(t[e]) + (r & mask)) & ~mask);
+        }
+      }
+      if (WT == W_BF16) {
+        uint2 o;
+        o.x = (unsigned)bf16_bits(t[0]) | ((unsigned)bf16_bits(t[1]) << 16);
+        o.y = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
+        *(uint2*)((unsigned short*)w + idx) = o;
+      } else {
+        int packed = 0;   // no clamp: torch's cast gives NaN above 464 and so does the converter
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
+        *(int*)((unsigned char*)w + idx) = packed;
+      }
+    }
+  }
+}
+
+}  // namespace xmc

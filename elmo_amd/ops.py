@@ -93,5 +93,56 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
     return out
 
 
+WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}
+
+
+def tiled_workspace_bytes(num_chunks, rows_per_chunk):
+    n = _lib.load().xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk)
+    if n == 0:
+        raise _lib.XmcError("unsupported chunk geometry")
+    return n
+
+
+def alloc_tiled_workspace(num_chunks, rows_per_chunk, device):
+    return torch.empty(tiled_workspace_bytes(num_chunks, rows_per_chunk), dtype=torch.uint8, device=device)
+
+
+def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=None, round_mode="rtn", workspace=None,
+               grad_out=None, want_f32=False):
+    """One training step of the bf16 layer (chunked.py:76-133) or of the simulated-FP8 mode of the FP8 layer
+    (chunked_fp8xmc_clf.py:98-99,110,115-116), three kernels per chunk.  `chunk_views` are contiguous [rows, 768]
+    tensors (views of one weight tensor, or the FP8 layer's chunk parameters): all have rows_per_chunk rows except the
+    last, which may be shorter.  Updated in place; returns grad_input (bf16) or (grad_input, grad_x_fp32)."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == FEATURES
+    assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
+    assert labels.dim() == 2 and labels.shape[1] == 2
+    assert round_mode in ("rtn", "sr_philox"), "the tiled path rounds to nearest or with the reference's Philox recipe"
+    wdt = (torch.bfloat16,) if weight_type == "bf16" else (torch.float8_e4m3fn, torch.uint8)
+    nc = len(chunk_views)
+    arr = (ctypes.c_void_p * nc)()
+    for i, c in enumerate(chunk_views):
+        assert c.is_cuda and c.is_contiguous() and c.dtype in wdt and c.dim() == 2 and c.shape[1] == FEATURES
+        assert c.shape[0] == rows_per_chunk or (i == nc - 1 and 0 < c.shape[0] <= rows_per_chunk)
+        arr[i] = c.data_ptr()
+    batch = x.shape[0]
+    assert 0 < batch <= MAX_BATCH, "batch must be at most 128"
+    if workspace is None:
+        workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device)
+    if grad_out is None:
+        grad_out = torch.empty(batch, FEATURES, dtype=torch.bfloat16, device=x.device)
+    gf = torch.empty(batch, FEATURES, dtype=torch.float32, device=x.device) if want_f32 else None
+    sarr = None
+    if seeds is not None:
+        sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
+    st = lib.xmc_tiled_step(arr, nc, rows_per_chunk, chunk_views[-1].shape[0], WEIGHT_TYPES[weight_type], x.data_ptr(),
+                            batch, FEATURES, labels.data_ptr() if labels.numel() else None, labels.shape[0], float(lr),
+                            sarr, _lib.ROUND_MODES[round_mode], grad_out.data_ptr(),
+                            gf.data_ptr() if gf is not None else None, workspace.data_ptr(), workspace.numel(),
+                            _stream_ptr())
+    _lib.check(st, "xmc_tiled_step")
+    return (grad_out, gf) if want_f32 else grad_out
+
+
 def step_error_word(workspace, num_chunks, rows_per_chunk):
     return _lib.load().xmc_step_error_word(workspace.data_ptr(), num_chunks, rows_per_chunk, _stream_ptr())

@@ -53,7 +53,6 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         features = cfg.model.xmc.input_features
         assert features == ops.FEATURES, f"the gfx950 kernels are built for {ops.FEATURES} input features"
         assert self.device.type == "cuda", "Fp8XMCBCEChunkedLayer needs a GPU device: there is no CPU path"
-        assert not self.fake_fp8_matmul, "training.xmc.simulated_fp8 is not implemented by this build"
 
         # same initialisation as the reference (:29-32): xavier-uniform on the padded fp32 matrix, cast per chunk
         xfc_weight = torch.empty(self.num_labels, features, dtype=torch.float32)
@@ -69,8 +68,9 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
             assert self.xfc_weight[i].shape[0] == self.num_labels_i
         assert n_labels == self.num_labels
 
-        self.rounding = _opt(cfg.training.xmc, "rounding", "sr_fast")
-        assert self.rounding in ("sr_fast", "sr_philox", "rtn")
+        # simulated FP8 (:98-99,115-116) runs on the three-kernel path, which rounds with the reference's recipe
+        self.rounding = _opt(cfg.training.xmc, "rounding", "sr_philox" if self.fake_fp8_matmul else "sr_fast")
+        assert self.rounding in (("sr_philox", "rtn") if self.fake_fp8_matmul else ("sr_fast", "sr_philox", "rtn"))
         self.scale_w = float(_opt(cfg.training.xmc, "scale_w", 1.0))
         self.scale_x = float(_opt(cfg.training.xmc, "scale_x", 1.0))
         self.block_size = 16
@@ -79,6 +79,10 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self.grad_input = None
         # all scratch memory of the step comes from the torch allocator (so that max_memory_allocated sees it)
         self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
+        self._tiled_workspace = None
+        if self.fake_fp8_matmul:
+            assert self.scale_w == 1.0 and self.scale_x == 1.0, "simulated FP8 has no per-tensor scales"
+            self._tiled_workspace = ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device)
 
     def _chunks(self):
         return [w.data for w in self.xfc_weight]
@@ -113,7 +117,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
             skip_loss: ignored, as in the reference's FP8 layer; the return value is 0.
         '''
         assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
-        assert embed.shape[0] % 16 == 0 and embed.shape[0] <= ops.MAX_BATCH, \
+        assert embed.shape[0] <= ops.MAX_BATCH and (self.fake_fp8_matmul or embed.shape[0] % 16 == 0), \
             "batch must be a multiple of 16 and at most 128 (the reference data loader uses drop_last)"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
         x = embed.detach()
@@ -125,8 +129,12 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         loss = 0
         # one seed per chunk from the global CPU generator, exactly as the reference draws them (:113)
         seeds = [torch.randint(0, 1000000, (1,)).item() for _ in range(self.num_chunks)]
-        self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
-                                       scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
+        if self.fake_fp8_matmul:
+            self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
+                                             round_mode=self.rounding, workspace=self._tiled_workspace)
+        else:
+            self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
+                                           scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
         self.iteration += 1
         return loss
 

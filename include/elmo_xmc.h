@@ -79,6 +79,32 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
  * then forgets them.  Pass nulls to cancel. */
 int xmc_profile_events(void* start_event, void* stop_event);
 
+/* weight types of the tiled path */
+enum {
+  XMC_WEIGHT_E4M3 = 0,      /* simulated-FP8 mode of the FP8 layer (chunked_fp8xmc_clf.py:98-99,110,115-116) */
+  XMC_WEIGHT_BF16 = 1       /* bf16 layer (chunked.py:85-131) */
+};
+
+/* Bytes of workspace xmc_tiled_step needs. */
+size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk);
+
+/* One training step of the modes in which the reference keeps bf16 temporaries, three kernels per chunk as there:
+ *   XMC_WEIGHT_BF16  XMCBCECHUNKEDLayer.xfc_forward_backward (chunked.py:76-133) with sgd_update
+ *                    (stochastic_rounding_kernel.py:91-99): bf16 logits, grad_X partial rounded to bf16 per chunk,
+ *                    grad_W rounded to bf16, W = SR16(W - lr*A) (XMC_ROUND_SR_PHILOX) or bf16(W - lr*A) (XMC_ROUND_RTN)
+ *   XMC_WEIGHT_E4M3  Fp8XMCBCEChunkedLayer with simulated_fp8 (chunked_fp8xmc_clf.py:98-99,110,115-116;
+ *                    fuse_kernel.py:184-199): logits from the un-quantised bf16 X, W = e4m3_torch(SR20(W - lr*A)),
+ *                    where the final cast does not saturate (NaN above 464)
+ *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
+ *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
+ *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
+ *   round_mode       XMC_ROUND_RTN or XMC_ROUND_SR_PHILOX; batch: 1..128, any value
+ */
+int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                   const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
+                   const uint32_t* seeds, int round_mode, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
 /* Selects the fused kernel that xmc_fp8_step launches (no counterpart in the reference): 0 = four compute units per
  * tile stream without repeated arithmetic (default), 1 = two compute units per tile stream with the logits computed
  * twice.  Both produce the same weights; grad_X differs by fp32 summation order only.  The environment variable

@@ -119,6 +119,7 @@ def test_error_convention(gpu):
         xfc.xfc_forward_backward(torch.randn(16, 512, device=gpu).to(torch.bfloat16), labels, [0.05])
     with pytest.raises(AssertionError):
         xfc.xfc_forward_backward(torch.randn(16, 768).to(torch.bfloat16), labels, [0.05])
+    with pytest.raises(AssertionError):      # the simulated mode has no fast stochastic rounding and no scales
+        build(gpu, 1000, 2, simulated=True, rounding="sr_fast")
     with pytest.raises(AssertionError):
-        build(gpu, 1000, 2, ) if False else __import__("xmc_classifiers.chunked_fp8xmc_clf", fromlist=["x"]).Fp8XMCBCEChunkedLayer(
-            make_cfg("cuda:0", 1000, 2, simulated=True))
+        build(gpu, 1000, 2, simulated=True, scale_w=0.5)

@@ -1,0 +1,201 @@
+"""Parity of the three-kernel path (bf16 layer and simulated-FP8 mode, through the C ABI) against the CPU oracle.
+
+Tolerances: round-to-nearest weights within 1 grid step (e4m3 step; bf16: one ulp of the operands of the update, see
+check_bf16_weights) of the oracle with all but a small fraction identical (the fp32 accumulators differ by summation order only); the reference's stochastic-rounding recipe
+bit-identical wherever the fp32 value T it rounds is, i.e. for all but the same small fraction; grad_X accumulator
+within 1e-3 of its largest entry, grad_input its round-to-nearest bf16 image."""
+import numpy as np
+import pytest
+
+import helpers as H
+from elmo_amd import synth
+from oracle import codecs as C
+from oracle import step as O
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_case(L, batch, seed, pos_mean=5.0):
+    x = synth.make_x(batch, 768, seed)
+    w = C.bf16_round(synth.make_weights_np(L, 768, seed, 0.02))
+    labels = synth.make_labels(batch, L, pos_mean, 1.0, seed).astype(np.int32)
+    return x, w, labels
+
+
+def run_bf16(x, w, labels, nc, device, mode, seeds, lr=0.05):
+    import torch
+    from elmo_amd import ops
+    L = w.shape[0]
+    cs = (L + nc - 1) // nc
+    wt = torch.from_numpy(C.bf16_bits(w).view(np.int16)).to(device).view(torch.bfloat16)
+    views = [wt[c * cs:min((c + 1) * cs, L)] for c in range(nc) if c * cs < L]
+    xt = torch.from_numpy(C.bf16_bits(x).view(np.int16)).to(device).view(torch.bfloat16)
+    lab = torch.from_numpy(labels).to(device).contiguous()
+    g, gf = ops.tiled_step(views, cs, "bf16", xt, lab, lr, seeds=seeds, round_mode=mode, want_f32=True)
+    return wt.float().cpu().numpy(), gf.cpu().numpy(), g.float().cpu().numpy()
+
+
+def check_bf16_weights(new, ref_w, w0, x=None, lr=0.05):
+    """Updated bf16 weights: identical except where the bf16 rounding of grad_W (chunked.py:119) or of the result flipped
+    because the fp32 sums were taken in another order.  Such a flip moves the weight by one bf16 ulp of lr*A or of the
+    result (the first can cause the second); each is bounded by 2^-7 (|w_old| + |w_new|), which also covers results next
+    to zero after cancellation.  A flip of one bf16 entry of G itself (one ulp of a sigmoid, at most 2^-8) moves a whole
+    row of grad_W by that times |x|: an absolute floor of lr * 2^-8 * max|x|, twice over."""
+    tol = 1.5 * 2.0 ** -7 * (np.abs(w0) + np.abs(ref_w)) + 1e-30
+    if x is not None:
+        tol = tol + 2.0 * lr * 2.0 ** -8 * np.abs(x).max()
+    assert np.all(np.abs(new - ref_w) <= tol), float(np.max(np.abs(new - ref_w) / tol))
+    assert (new != ref_w).mean() < 2e-3, (new != ref_w).mean()
+
+
+def check_gx(gf, gb, ref_gx, tol=1e-3):
+    scale = np.abs(ref_gx).max()
+    assert np.abs(gf - ref_gx).max() <= tol * scale
+    assert np.array_equal(C.bf16_bits(gb), C.bf16_bits(C.bf16_round(gf)))
+
+
+@pytest.mark.parametrize("L,nc,batch,seed", [
+    (64, 1, 16, 31),            # a single tile
+    (1000, 3, 24, 32),          # ragged chunks (334, 334, 332), batch not a multiple of 16
+    (5000, 2, 128, 33),         # full batch
+    (20011, 4, 64, 34),         # prime label count
+])
+def test_bf16_layer_rtn_parity(gpu, L, nc, batch, seed):
+    x, w, labels = bf16_case(L, batch, seed)
+    new, gf, gb = run_bf16(x, w, labels, nc, gpu, "rtn", None)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.05, nc, sr_mode="rtn")
+    check_bf16_weights(new, ref_w, w, x)
+    # the per-chunk partial is rounded to bf16 before it is accumulated (chunked.py:116): a flip of that rounding moves
+    # an entry by one bf16 ulp of the partial, hence the looser bound
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+
+
+def test_bf16_layer_reference_stochastic_rounding(gpu):
+    L, nc, batch = 3000, 3, 32
+    x, w, labels = bf16_case(L, batch, 41)
+    seeds = [12345, 999999, 7]
+    new, gf, gb = run_bf16(x, w, labels, nc, gpu, "sr_philox", seeds)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.05, nc, seeds=seeds, sr_mode="reference")
+    check_bf16_weights(new, ref_w, w, x)
+    # stochastic rounding really happened: differs from round-to-nearest in a sizeable share of the weights
+    rtn_w, _, _ = O.bf16_step(w, x, labels, 0.05, nc, sr_mode="rtn")
+    assert (new != rtn_w).mean() > 0.2
+    # a different seed gives a different result
+    new2, _, _ = run_bf16(x, w, labels, nc, gpu, "sr_philox", [1, 2, 3])
+    assert (new2 != new).mean() > 0.1
+
+
+def test_bf16_layer_duplicates_and_no_positives(gpu):
+    x, w, labels = bf16_case(640, 16, 51)
+    dup = np.array([[0, 5], [0, 5], [3, 639], [3, 639], [15, 0]], dtype=np.int32)
+    new, gf, gb = run_bf16(x, w, dup, 2, gpu, "rtn", None)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, dup, 0.05, 2, sr_mode="rtn")
+    check_bf16_weights(new, ref_w, w, x)
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+    none = np.zeros((0, 2), dtype=np.int32)
+    new, gf, gb = run_bf16(x, w, none, 2, gpu, "rtn", None)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, none, 0.05, 2, sr_mode="rtn")
+    check_bf16_weights(new, ref_w, w, x)
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+
+
+def run_sim(case, device, mode, seeds, lr=0.05):
+    from elmo_amd import ops
+    chunks, x, labels = H.to_device_case(case, device)
+    g, gf = ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", x, labels, lr, seeds=seeds, round_mode=mode, want_f32=True)
+    return H.chunks_to_numpy(chunks), gf.cpu().numpy(), g.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("nc,rows,batch,seed", [(1, 64, 16, 61), (3, 208, 32, 62), (2, 4096, 128, 63)])
+def test_simulated_fp8_rtn_parity(gpu, nc, rows, batch, seed):
+    case = H.make_case(nc, rows, batch, seed)
+    new, gf, gb = run_sim(case, gpu, "rtn", None)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn", simulated=True)
+    mism = total = 0
+    for a, b in zip(new, ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1
+        mism += int((d != 0).sum()); total += d.size
+    assert mism / total < 2e-3
+    check_gx(gf, gb, ref_gx)
+
+
+def test_simulated_fp8_differs_from_true_fp8_logits(gpu):
+    """The simulated mode takes its logits from the un-quantised X (chunked_fp8xmc_clf.py:99): its grad_X must match the
+    simulated oracle and not the true-FP8 one."""
+    case = H.make_case(2, 1024, 32, 64)
+    _, gf, _ = run_sim(case, gpu, "rtn", None)
+    _, gx_sim, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn", simulated=True)
+    _, gx_true, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn", simulated=False)
+    assert np.abs(gf - gx_sim).max() < 0.2 * np.abs(gx_true - gx_sim).max()
+
+
+def test_simulated_fp8_reference_stochastic_rounding_and_overflow(gpu):
+    case = H.make_case(2, 512, 32, 65)
+    seeds = [424242, 17]
+    new, gf, gb = run_sim(case, gpu, "sr_philox", seeds)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, seeds=seeds, sr_mode="reference",
+                                      simulated=True)
+    mism = total = 0
+    for a, b in zip(new, ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1
+        mism += int((d != 0).sum()); total += d.size
+    assert mism / total < 2e-3
+    # the cast back to e4m3 does not saturate (torch semantics, :116): a weight pushed beyond 464 becomes NaN
+    big = H.make_case(1, 64, 16, 66)
+    big["chunks"][0][:] = 0x7E                     # +448 everywhere
+    big["labels"] = np.array([[b, l] for b in range(16) for l in range(8)], dtype=np.int32)
+    new, _, _ = run_sim(big, gpu, "rtn", None, lr=2000.0)
+    ref_codes, _, _ = O.fp8_step(big["chunks"], big["x"], big["labels"], 2000.0, sr_mode="rtn", simulated=True)
+    assert np.array_equal(new[0] & 0x7F == 0x7F, ref_codes[0] & 0x7F == 0x7F) and (new[0] & 0x7F == 0x7F).any()
+
+
+def test_chunked_module_contract(gpu):
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked import XMCBCECHUNKEDLayer
+    cfg = make_cfg("cuda:0", 1000, 3, rounding="rtn")
+    cfg.model.xmc.dtype = "bfloat16"
+    torch.manual_seed(0)
+    xfc = XMCBCECHUNKEDLayer(cfg)
+    assert xfc.xfc_weight.shape == (1000, 768) and xfc.xfc_weight.dtype == torch.bfloat16 and xfc.chunk_size == 334
+    assert list(xfc.state_dict().keys()) == []            # a plain tensor attribute, as in the reference
+    enc = torch.nn.Linear(768, 768, bias=False).to(gpu).to(torch.bfloat16)
+    tokens = torch.randn(24, 768, device=gpu, dtype=torch.bfloat16)
+    labels = torch.tensor([[0, 3], [0, 999], [5, 17], [23, 500], [23, 500]], dtype=torch.int32, device=gpu)
+    w0 = xfc.xfc_weight.float().cpu().numpy()
+    ptr = xfc.xfc_weight.data_ptr()
+    out = enc(tokens)
+    loss = xfc.xfc_forward_backward(out, labels, [0.05], skip_loss=True)
+    assert loss == 0 and xfc.iteration == 1 and xfc.xfc_weight.data_ptr() == ptr
+    g = xfc.grad_input
+    assert g.shape == (24, 768) and g.dtype == torch.bfloat16
+    ref_w, ref_gx, _ = O.bf16_step(w0, out.detach().float().cpu().numpy(), labels.cpu().numpy(), 0.05, 3, sr_mode="rtn")
+    check_bf16_weights(xfc.xfc_weight.float().cpu().numpy(), ref_w, w0, out.detach().float().cpu().numpy())
+    out.backward(g[0:24, :])
+    assert enc.weight.grad is not None
+    logits = xfc.xfc_forward(tokens)
+    assert logits.shape == (24, 1000)
+    with pytest.raises(AssertionError):
+        cfg2 = make_cfg("cuda:0", 1000, 3)
+        cfg2.model.xmc.dtype = "float32"
+        XMCBCECHUNKEDLayer(cfg2)
+
+
+def test_fp8_module_simulated_mode(gpu):
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked_fp8xmc_clf import Fp8XMCBCEChunkedLayer
+    torch.manual_seed(0)
+    xfc = Fp8XMCBCEChunkedLayer(make_cfg("cuda:0", 1000, 2, simulated=True, rounding="rtn"))
+    tokens = torch.randn(32, 768, device=gpu, dtype=torch.bfloat16) * 0.05
+    labels = torch.tensor([[0, 3], [31, 999]], dtype=torch.int32, device=gpu)
+    before = [w.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    assert xfc.xfc_forward_backward(tokens, labels, [0.05]) == 0
+    ref_codes, ref_gx, _ = O.fp8_step(before, tokens.float().cpu().numpy(), labels.cpu().numpy(), 0.05, sr_mode="rtn",
+                                      simulated=True)
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        d = H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r)
+        assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    assert xfc.grad_input.shape == (32, 768)
