@@ -368,7 +368,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     issue_mailbox(i);
     QT(2)
 
-    stage_a(i + QAHEAD, inf[QAHEAD]);
+    // The two wavefronts of a SIMD run stage A and grad_X in opposite orders, so that the LDS reads of one overlap
+    // the MFMAs of the other.  The stores of stage A stay ahead of the weight stores in both orders (see the wait above).
+    if (h == 0) stage_a(i + QAHEAD, inf[QAHEAD]);
     QT(3)
 
     // ---- grad_X[64 x 48] += G^T W; 6 steps (32-row K step major, 16-feature block minor); the transposed W read of
@@ -398,6 +400,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
           acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[ks2][mb], wb[s & 1], acc2[mb][nn], 0, 0, 0);
       }
     }
+    if (h != 0) stage_a(i + QAHEAD, inf[QAHEAD]);
     QT(4)
 
     // ---- A^T[48 features x 32 rows] = X^T G^T in two 16-row blocks, each followed by its update.  Row r = 4kg+e of
