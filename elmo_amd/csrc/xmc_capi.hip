@@ -30,6 +30,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
     (void)hipFuncSetAttribute((const void*)sort_keys_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
+    (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
   }
   return cached[dev];
 }
@@ -121,12 +122,12 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   int n_pad = 0;
   if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
 
-  (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
-  if (n_pad > 0)
-    sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
-  tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
-                                                                tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
   if (step_kernel_choice() == 1) {
+    (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
+    if (n_pad > 0)
+      sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
+    tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
+                                                                  tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
     prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                                 (unsigned short*)(ws + WS_XT));
     StepParams p;
@@ -158,8 +159,6 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     reduce_gx_kernel<<<96, NT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), grid, scale_w, grad_x_f32,
                                            (unsigned short*)grad_x_bf16, batch);
   } else {
-    prep_x_quad_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x,
-                                                                     ws + WS_XQ, (unsigned short*)(ws + WS_XT));
     QuadParams p;
     for (int c = 0; c < MAX_CHUNKS; c++) {
       p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
@@ -183,7 +182,12 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.batch = batch;
     const int qgrid = grid / 32 * 32;   // whole quads on every XCD
     if (qgrid < 32) return XMC_ERR_DEVICE;
-    tile_desc_kernel<<<(num_tiles + 255) / 256, 256, 0, stream>>>(p, desc);
+    quad_sort_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS),
+                                                            (int*)(ws + WS_FLAGS));
+    const int desc_blocks = (num_tiles + 1 + 255) / 256;
+    quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, 0, stream>>>(
+        p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
+        (unsigned short*)(ws + WS_XT));
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
     switch (round_mode) {
       case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;

@@ -132,16 +132,87 @@ __device__ __forceinline__ QTile q_from_desc(uint4 d0, uint4 d1) {
   return q;
 }
 
-// desc[t] = {base pointer, seed, first key | one past last key, row in chunk, valid rows, first label}
-__global__ void tile_desc_kernel(const QuadParams p, uint4* desc) {
-  int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= p.num_tiles) return;
-  const int c = t / p.tiles_per_chunk;
-  const int row0 = (t - c * p.tiles_per_chunk) * TL;
-  const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
-  desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), p.seed[c], (unsigned)p.tile_ptr[t]};
-  desc[2 * t + 1] = uint4{(unsigned)p.tile_ptr[t + 1], (unsigned)row0, (unsigned)min(TL, p.rows_per_chunk - row0),
-                          (unsigned)(c * p.rows_per_chunk + row0)};
+// First of the two launches in front of the step kernel (single workgroup): clear the counters and sort the positives
+// (key = label*256 + batch row, invalid entries -> 0xFFFFFFFF).  Up to 2048 keys are sorted by rank - every thread counts
+// the keys that precede its own, one pass over LDS with no barriers in between - larger sets by a bitonic network.
+__global__ __launch_bounds__(1024) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys, int* flags) {
+  extern __shared__ unsigned sk[];
+  const int tid = threadIdx.x;
+  flags[tid] = 0;
+  for (int i = tid; i < n_pad; i += 1024) {
+    unsigned key = 0xFFFFFFFFu;
+    if (i < nnz) {
+      int r = coo[2 * i], l = coo[2 * i + 1];
+      if (r >= 0 && r < batch && l >= 0 && l < (1 << 24) - 1) key = ((unsigned)l << 8) | (unsigned)r;
+    }
+    sk[i] = key;
+  }
+  __syncthreads();
+  if (n_pad <= 2048) {
+    for (int i = tid; i < n_pad; i += 1024) {
+      const unsigned mine = sk[i];
+      int rank = 0;
+      for (int j = 0; j < n_pad; j++) {
+        const unsigned o = sk[j];
+        rank += (o < mine || (o == mine && j < i)) ? 1 : 0;
+      }
+      keys[rank] = mine;
+    }
+    return;
+  }
+  for (int k = 2; k <= n_pad; k <<= 1) {
+    for (int jj = k >> 1; jj > 0; jj >>= 1) {
+      for (int i = tid; i < n_pad; i += 1024) {
+        int ixj = i ^ jj;
+        if (ixj > i) {
+          unsigned a = sk[i], b = sk[ixj];
+          bool up = (i & k) == 0;
+          if ((a > b) == up) { sk[i] = b; sk[ixj] = a; }
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < n_pad; i += 1024) keys[i] = sk[i];
+}
+
+__device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
+                                                   unsigned short* xt);
+
+// Second launch: blocks below desc_blocks write, for every tile,
+//   desc[t] = {base pointer, seed, first key | one past last key, row in chunk, valid rows, first label}
+//   tile_ptr[t] = first key whose label >= first label of tile t (binary search in the sorted keys)
+// and the remaining blocks build the operand images of X.
+__global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p, int n_pad, int* tile_ptr, uint4* desc, int desc_blocks,
+                                                             const unsigned short* x, float inv_scale_x, unsigned char* xq,
+                                                             unsigned short* xt) {
+  if ((int)blockIdx.x >= desc_blocks) {
+    prep_x_quad_thread(((int)blockIdx.x - desc_blocks) * 256 + (int)threadIdx.x, x, p.batch, inv_scale_x, xq, xt);
+    return;
+  }
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t > p.num_tiles) return;
+  auto lower = [&](int tt) {   // first key of tile tt (tt == num_tiles: first key past the last tile)
+    const int c = tt / p.tiles_per_chunk, tj = tt - c * p.tiles_per_chunk;
+    const unsigned long long bound = ((unsigned long long)c * p.rows_per_chunk + (unsigned long long)tj * TL) << 8;
+    int lo = 0, hi = n_pad;
+    while (lo < hi) {
+      int mid = (lo + hi) >> 1;
+      if ((unsigned long long)p.keys[mid] < bound) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+  };
+  const int p0 = lower(t);
+  tile_ptr[t] = p0;
+  if (t < p.num_tiles) {
+    const int p1 = lower(t + 1);
+    const int c = t / p.tiles_per_chunk;
+    const int row0 = (t - c * p.tiles_per_chunk) * TL;
+    const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
+    desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), p.seed[c], (unsigned)p0};
+    desc[2 * t + 1] = uint4{(unsigned)p1, (unsigned)row0, (unsigned)min(TL, p.rows_per_chunk - row0),
+                            (unsigned)(c * p.rows_per_chunk + row0)};
+  }
 }
 
 template <int MODE>
@@ -471,10 +542,15 @@ __global__ __launch_bounds__(QNT) void reduce_gx_quad_kernel(const floatx4* part
   const int slot = blockIdx.x >> 2, m = blockIdx.x & 3;   // slot = mb*3+nn
   const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fg = v & 3, h = v >> 2;
+  // the workgroups of member m, in a fixed order; eight loads in flight at a time
   floatx4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int g = 0; g < nwg; g++) {
-    if (((g >> 3) & 3) != m) continue;
-    s += partial[((size_t)g * 12 + slot) * QNT + tid];
+  const int nq = nwg >> 5;   // quads per XCD
+  for (int jq = 0; jq < nq; jq++) {
+    floatx4 v[8];
+#pragma unroll
+    for (int x = 0; x < 8; x++) v[x] = partial[((size_t)(((jq * 4 + m) << 3) + x) * 12 + slot) * QNT + tid];
+#pragma unroll
+    for (int x = 0; x < 8; x++) s += v[x];
   }
   const int mb = slot / 3, nn = slot - mb * 3;
   const int col = QCOLS * m + 48 * fg + 16 * nn + l16;
@@ -494,8 +570,9 @@ __global__ __launch_bounds__(QNT) void reduce_gx_quad_kernel(const floatx4* part
 //       byte j: Xq[b][k = 128ks + 32kg + j]
 //   xt: bf16 X^T in v_mfma 16x16x32 A-operand order: [((col/48)*3 + cg)*4 + ks][lane][8 bf16], lane = r + 16*kg,
 //       element j = X[32ks + 8kg + j][col] with col = 48*(col/48) + 12*(r/4) + 4*cg + r%4
-__global__ void prep_x_quad_kernel(const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq, unsigned short* xt) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (b, group of 4 features)
+__device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
+                                                   unsigned short* xt) {
+  // one thread per (b, group of 4 features)
   if (i >= BP * (D / 4)) return;
   int b = i / (D / 4), k = (i - b * (D / 4)) * 4;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
