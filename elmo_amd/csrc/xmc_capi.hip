@@ -240,9 +240,13 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk) {
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
                    const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
-                   const uint32_t* seeds, int round_mode, void* grad_x_bf16, float* grad_x_f32, void* workspace,
-                   size_t workspace_bytes, void* stream_) {
+                   const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                   int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes,
+                   void* stream_) {
   if (!chunk_ptrs || !x_bf16 || !workspace || !grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
+  if (kahan_type < 0 || kahan_type > 2 || (kahan_type != 0 && (weight_type != W_E4M3 || !kahan))) return XMC_ERR_MODE;
+  if (kahan_type != 0 && (num_head < 0 || num_head > rows_per_chunk || !aligned16(kahan))) return XMC_ERR_SHAPE;
+  if (kahan_type == 0) num_head = 0;
   if (features != D || batch <= 0 || batch > BP) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_last_chunk <= 0 || rows_last_chunk > rows_per_chunk) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
@@ -278,7 +282,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (n_pad > 0)
     sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys);
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
-  tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, xb, xT);
+  tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, quantize_x, xb, xT);
   tiled_zero_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>(gx_total, BP * D);
   for (int c = 0; c < num_chunks; c++) {
     void* w = chunk_ptrs[c];
@@ -287,6 +291,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int tiles = rp / TL;
     const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;
     const unsigned seed = seeds ? seeds[c] : 0u;
+    const int nh = c == 0 ? num_head : 0;   // the compensated head lives in chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127)
     int range = (rp + T_SPLITS - 1) / T_SPLITS;
     range = (range + TL - 1) / TL * TL;
     const int splits = (rp + range - 1) / range;
@@ -299,11 +304,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     }
     tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total);
     if (weight_type == W_BF16) {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
-      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
     } else {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
-      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed);
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
     }
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);

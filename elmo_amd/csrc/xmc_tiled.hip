@@ -39,13 +39,21 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
   return t_fp8x8_to_bf16x8(*(const intx2*)((const unsigned char*)w + idx));
 }
 
-// X -> zero-padded row-major image and its transpose
-__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, unsigned short* xb, unsigned short* xT) {
+// X -> zero-padded row-major image (for the logits; optionally quantised to e4m3 and widened back, which makes the bf16
+// products equal to the FP8 ones of chunked_fp8xmc_clf.py:101-102) and its transpose (for grad_W, never quantised)
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int quantize, unsigned short* xb, unsigned short* xT) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= BP * D) return;
   int b = i / D, k = i - b * D;
   unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
-  xb[i] = v;
+  unsigned short vq = v;
+  if (quantize) {
+    const float f = clamp448(bf16_from_bits(v));
+    const int code = __builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false);
+    const floatx2 back = __builtin_amdgcn_cvt_pk_f32_fp8(code, false);
+    vq = bf16_bits(back.x);
+  }
+  xb[i] = vq;
   xT[(size_t)k * BP + b] = v;
 }
 
@@ -210,10 +218,15 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 //      of the tile and features 192fb.. (12 blocks of 16).  A^T[f][l] = sum_b X^T[f][b] G[l][b]; a lane ends up with four
 //      consecutive features of one label row.
 //        bf16 weights : a = bf16(A); t = w - lr*a; RTN: bf16(t);  SR: bits(t) + (philox(seed, l*768+f) & 0xFFFF), clear 16 bits
-//        e4m3 weights : t = w - lr*A;          RTN: e4m3(t) as torch casts (NaN above 464); SR: add 20 bits, clear, same cast
+//        e4m3 weights : t = w - lr*A;          RTN: e4m3(t); SR: add 20 bits, clear, same cast.  The cast is torch's (NaN above
+//                       464; simulated FP8, chunked_fp8xmc_clf.py:116) or saturating at +-448 (true FP8, fuse_kernel.py:35).
+//        head-Kahan (e4m3 weights, rows below num_head; fuse_kernel.py:202-262): t = (w + k) - lr*A, W' = round(t),
+//                       k' = ((k + w) - W') - lr*A stored as bf16 (kahan_type 1) or e5m2 (2); rows behind the head take
+//                       their random offsets from (row - num_head), as the reference's call on the sliced tensors does
 template <int WT, int MODE>
 __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, const unsigned short* xT,
-                                                           float lr, unsigned seed) {
+                                                           float lr, unsigned seed, int saturate, void* kahan, int kahan_type,
+                                                           int num_head) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, tile = blockIdx.x >> 2;
   const int row = tile * TL + 16 * wv + l16;
@@ -243,13 +256,27 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
         floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, true);
         wv4[0] = w01.x; wv4[1] = w01.y; wv4[2] = w23.x; wv4[3] = w23.y;
       }
+      const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
+      const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
+      float kv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (head) {
+        if (kahan_type == 1) {
+          const uint2 raw = *(const uint2*)((const unsigned short*)kahan + idx);
+          kv[0] = bf16_from_bits((unsigned short)(raw.x & 0xffffu)); kv[1] = bf16_from_bits((unsigned short)(raw.x >> 16));
+          kv[2] = bf16_from_bits((unsigned short)(raw.y & 0xffffu)); kv[3] = bf16_from_bits((unsigned short)(raw.y >> 16));
+        } else {
+          const int raw = *(const int*)((const unsigned char*)kahan + idx);
+          floatx2 k01 = __builtin_amdgcn_cvt_pk_f32_bf8(raw, false), k23 = __builtin_amdgcn_cvt_pk_f32_bf8(raw, true);
+          kv[0] = k01.x; kv[1] = k01.y; kv[2] = k23.x; kv[3] = k23.y;
+        }
+      }
       float t[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         const float g = WT == W_BF16 ? bf16_rt(a[e]) : a[e];
-        t[e] = __builtin_fmaf(-lr, g, wv4[e]);
+        t[e] = __builtin_fmaf(-lr, g, head ? wv4[e] + kv[e] : wv4[e]);
         if (MODE == ROUND_SR_PHILOX) {
-          const unsigned r = philox_word0((unsigned)row * (unsigned)D + (unsigned)(col + e), seed, 0u);
+          const unsigned r = philox_word0((unsigned)orow * (unsigned)D + (unsigned)(col + e), seed, 0u);
           const unsigned mask = WT == W_BF16 ? 0xFFFFu : 0xFFFFFu;
           t[e] = __uint_as_float((__float_as_uint(t[e]) + (r & mask)) & ~mask);
         }
@@ -260,10 +287,34 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
         o.y = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
         *(uint2*)((unsigned short*)w + idx) = o;
       } else {
-        int packed = 0;   // no clamp: torch's cast gives NaN above 464 and so does the converter
+        if (saturate) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) t[e] = clamp448(t[e]);
+        }
+        int packed = 0;   // without the clamp: torch's cast gives NaN above 464 and so does the converter
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
         packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
         *(int*)((unsigned char*)w + idx) = packed;
+        if (head) {
+          floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, true);
+          const float wn[4] = {n01.x, n01.y, n23.x, n23.y};
+          float kn[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) kn[e] = __builtin_fmaf(-lr, a[e], (kv[e] + wv4[e]) - wn[e]);
+          if (kahan_type == 1) {
+            uint2 o;
+            o.x = (unsigned)bf16_bits(kn[0]) | ((unsigned)bf16_bits(kn[1]) << 16);
+            o.y = (unsigned)bf16_bits(kn[2]) | ((unsigned)bf16_bits(kn[3]) << 16);
+            *(uint2*)((unsigned short*)kahan + idx) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
+            int pk = 0;
+            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
+            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
+            *(int*)((unsigned char*)kahan + idx) = pk;
+          }
+        }
       }
     }
   }

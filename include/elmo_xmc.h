@@ -99,11 +99,18 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk);
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
  *   round_mode       XMC_ROUND_RTN or XMC_ROUND_SR_PHILOX; batch: 1..128, any value
+ *   quantize_x       e4m3 weights: 0 = logits from the un-quantised X (simulated FP8), 1 = from e4m3(X) (true FP8, :101)
+ *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
+ *   kahan, kahan_type, num_head
+ *                    head-Kahan update of Fp8XMCBCEChunkedHeadKahanLayer (chunked_head_kahan_fp8xmc_clf.py:41-48,127-131;
+ *                    fuse_kernel.py:202-262), e4m3 weights only: device buffer [num_head, 768] of bf16 (kahan_type 1) or
+ *                    e5m2 (kahan_type 2) for the first num_head rows of chunk 0, updated in place; kahan_type 0 = none
  */
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
                    const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
-                   const uint32_t* seeds, int round_mode, void* grad_x_bf16, float* grad_x_f32, void* workspace,
-                   size_t workspace_bytes, void* stream);
+                   const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                   int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes,
+                   void* stream);
 
 /* Selects the fused kernel that xmc_fp8_step launches (no counterpart in the reference): 0 = four compute units per
  * tile stream without repeated arithmetic (default), 1 = two compute units per tile stream with the logits computed

@@ -88,6 +88,42 @@ def e4m3_encode(x, saturate=True):
     return (code | sign).astype(np.uint8).reshape(x.shape)
 
 
+# --------------------------------------------------------------------------- e5m2 (OCP FP8, the Kahan buffer option)
+def e5m2_decode(codes):
+    """uint8 e5m2 codes -> fp32 (exact): the top byte of an IEEE half."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.uint16) << np.uint16(8)
+    return c.view(np.float16).astype(np.float32)
+
+
+def e5m2_encode(x, saturate=True):
+    """fp32 -> e5m2 code, round to nearest even (1-5-2, bias 15, max normal 57344, subnormal step 2^-16).
+    saturate=True: finite overflow and inf -> +-57344 (the satfinite conversion of the compiled kernels,
+    fuse_kernel.py:255); saturate=False: torch.Tensor.to(torch.float8_e5m2) semantics (overflow -> inf)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    a = np.abs(x).astype(np.float64)
+    sign = ((x.view(np.uint32) >> 31).astype(np.uint8) << 7).astype(np.uint8)
+    nan = np.isnan(x)
+    a = np.where(nan, 0.0, a)
+    if saturate:
+        a = np.minimum(a, 57344.0)
+    _, ex = np.frexp(a)
+    e = np.maximum(ex - 1, -14)
+    quantum = np.ldexp(1.0, e - 2)
+    val = np.rint(a / quantum) * quantum
+    over = val > 57344.0
+    _, ex2 = np.frexp(np.where(over, 1.0, val))
+    e2 = ex2 - 1
+    is_sub = val < 2.0 ** -14
+    exp_field = np.where(is_sub, 0, e2 + 15).astype(np.int64)
+    man = np.where(is_sub, val * 65536.0, (val / np.ldexp(1.0, e2) - 1.0) * 4.0)
+    man = np.where(val == 0, 0, man).astype(np.int64)
+    code = ((exp_field << 2) | man).astype(np.uint8)
+    code = np.where(val == 0, 0, code).astype(np.uint8)
+    code = np.where(over, 0x7C, code).astype(np.uint8)          # inf
+    code = np.where(nan, 0x7F, code).astype(np.uint8)
+    return (code | sign).astype(np.uint8).reshape(x.shape)
+
+
 # --------------------------------------------------------------------------- Philox-4x32-10
 _PH_M0 = np.uint64(0xD2511F53)
 _PH_M1 = np.uint64(0xCD9E8D57)

@@ -108,6 +108,64 @@ def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulate
     return out + (parts,) if return_parts else out
 
 
+def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="bf16", seeds=None, sr_mode="rtn"):
+    """One step of the head-Kahan FP8 layer (chunked_head_kahan_fp8xmc_clf.py:95-133; fuse_kernel.py:202-262), true FP8.
+
+    Logits, G and grad_X exactly as fp8_step.  Update of chunk 0 (:127-131): rows [0, num_head) carry a compensation
+    buffer `kahan` [num_head, d] (bf16 values or e5m2 codes):
+        w  = (f32(W) + f32(k)) - lr*A          (two fp32 roundings, the second one fused)
+        Wq = e4m3_sat(SR20(w))  or e4m3_sat(w) in "rtn" mode
+        k' = cast( ((f32(k) + f32(W)) - f32(Wq)) - lr*A )
+    with random offsets row*d + col; the remaining rows of chunk 0 are updated by a call on the sliced tensors, so
+    their offsets restart at zero: (row - num_head)*d + col.  Other chunks as in fp8_step.
+    Returns (new_codes list, new_kahan, gx_fp32, grad_input)."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.float32)
+    B, d = x.shape
+    nc, Lc = len(w_codes), w_codes[0].shape[0]
+    assert 0 <= num_head <= Lc
+    lr64 = float(np.float32(lr))
+    xq64 = C.e4m3_decode(C.e4m3_encode(x, saturate=True)).astype(np.float64)
+    x64 = x.astype(np.float64)
+    gx = np.zeros((B, d), dtype=np.float64)
+    k_old = (C.e5m2_decode(kahan) if kahan_type == "e5m2" else np.asarray(kahan, dtype=np.float32)).astype(np.float32)
+    new_codes, new_kahan = [], None
+
+    def rnd(t, seed, offs):
+        if sr_mode == "rtn":
+            return C.e4m3_encode(t, saturate=True)
+        return C.e4m3_encode(C.sr_add_mask(t, C.tl_randint(seed, offs), 20), saturate=True)
+
+    for c in range(nc):
+        w = C.e4m3_decode(w_codes[c])
+        w64 = w.astype(np.float64)
+        z = (w64 @ xq64.T).astype(np.float32)
+        pos = _positives_mask(labels, B, c * Lc, (c + 1) * Lc)
+        _, g = _grad_from_logits(z, pos)
+        g64 = g.astype(np.float64)
+        gx += g64.T @ w64
+        a = (g64 @ x64).astype(np.float32)
+        seed = None if seeds is None else seeds[c]
+        codes = np.empty_like(w_codes[c])
+        cols = np.arange(d, dtype=np.int64)[None, :]
+        lo = num_head if c == 0 else 0
+        if c == 0 and num_head > 0:
+            ah, wh = a[:num_head].astype(np.float64), w[:num_head]
+            s = (wh + k_old).astype(np.float32)                                     # weights + kahan
+            t = (s.astype(np.float64) - lr64 * ah).astype(np.float32)               # - lr*acc
+            offs = np.arange(num_head, dtype=np.int64)[:, None] * d + cols
+            codes[:num_head] = rnd(t, seed, offs)
+            wq = C.e4m3_decode(codes[:num_head])
+            u = ((k_old + wh).astype(np.float32) - wq).astype(np.float32)           # kahan + old - new
+            kn = (u.astype(np.float64) - lr64 * ah).astype(np.float32)              # - lr*acc
+            new_kahan = C.e5m2_encode(kn, saturate=True) if kahan_type == "e5m2" else C.bf16_round(kn)
+        t = (w64[lo:] - lr64 * a[lo:].astype(np.float64)).astype(np.float32)
+        offs = np.arange(Lc - lo, dtype=np.int64)[:, None] * d + cols
+        codes[lo:] = rnd(t, seed, offs)
+        new_codes.append(codes)
+    gx32 = gx.astype(np.float32)
+    return new_codes, new_kahan, gx32, C.bf16_round(gx32)
+
+
 def fp8_forward(w_codes, x_any, num_labels, *, simulated=False, scale_w=1.0, scale_x=1.0):
     """Inference logits [B, num_labels] (bf16-valued fp32): chunked_fp8xmc_clf.py:45-60.  The caller passes X
     already cast to e4m3 (evaluate.py:155-156); here X is re-quantised, which is idempotent."""

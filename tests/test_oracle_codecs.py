@@ -142,3 +142,23 @@ def test_sr_exact_agrees_with_hardware_converter_observations():
     for v, r, code in obs:
         got = int(C.sr_e4m3_exact(np.array([v], dtype=np.float32), np.array([r], dtype=np.uint64))[0])
         assert got == code, (v, hex(r), hex(got), hex(code))
+
+
+def test_e5m2_codec_matches_torch():
+    """e5m2 codes decode as the top byte of an IEEE half; the encoder equals torch's cast wherever torch stays finite and
+    saturates at 57344 where the compiled kernels do."""
+    codes = np.arange(256, dtype=np.uint8)
+    ref = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    got = C.e5m2_decode(codes)
+    assert np.array_equal(np.isnan(ref), np.isnan(got)) and np.array_equal(ref[~np.isnan(ref)], got[~np.isnan(got)])
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(100000).astype(np.float32) * np.float32(10.0) ** rng.integers(-7, 5, 100000),
+                        np.array([0.0, -0.0, 2.0 ** -16, 2.0 ** -17, 3 * 2.0 ** -17, 57344.0, 61439.0, 1.25, 1.375, 1.125],
+                                 dtype=np.float32)]).astype(np.float32)
+    t = torch.from_numpy(x).to(torch.float8_e5m2)
+    ref_codes = t.view(torch.uint8).numpy()
+    finite = np.isfinite(t.float().numpy())
+    assert np.array_equal(C.e5m2_encode(x, saturate=False)[finite], ref_codes[finite])
+    assert np.array_equal(C.e5m2_encode(x, saturate=False), ref_codes)                  # overflow -> inf as torch
+    big = np.array([61440.0, 1e6, np.inf, -1e9], dtype=np.float32)
+    assert np.array_equal(C.e5m2_decode(C.e5m2_encode(big, saturate=True)), np.array([57344.0, 57344.0, 57344.0, -57344.0], np.float32))

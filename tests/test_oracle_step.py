@@ -139,3 +139,38 @@ def test_example_shape_of_the_reference_smoke_function():
     # grad_X against a plain fp32 library GEMM on the same G
     ref = (torch.from_numpy(g).t() @ torch.from_numpy(C.e4m3_decode(w))).numpy()
     assert np.allclose(gx, ref, rtol=1e-3, atol=1e-3)
+
+
+def test_kahan_step_invariants():
+    """Head-Kahan update (fuse_kernel.py:202-262): with num_head = 0 it is the plain step; for head rows the buffer holds
+    what the rounding dropped, W' + k' = W + k - lr*A up to the rounding of k' itself; rows behind the head restart the
+    random offsets at zero; over repeated steps with a constant small gradient the compensated weights follow the exact
+    trajectory while round-to-nearest alone stalls."""
+    case = H.make_case(2, 64, 16, 71)
+    x, labels = case["x"], case["labels"]
+    ref = O.fp8_step(case["chunks"], x, labels, 0.05, sr_mode="rtn")
+    k0 = np.zeros((0, 768), dtype=np.float32)
+    codes, kn, gx, _ = O.fp8_kahan_step(case["chunks"], k0, x, labels, 0.05, 0, sr_mode="rtn")
+    assert all(np.array_equal(a, b) for a, b in zip(codes, ref[0])) and np.array_equal(gx, ref[1]) and kn is None
+    nh = 32
+    k0 = C.bf16_round(np.random.default_rng(1).standard_normal((nh, 768)).astype(np.float32) * 1e-3)
+    codes, kn, gx, _ = O.fp8_kahan_step(case["chunks"], k0, x, labels, 0.05, nh, sr_mode="rtn")
+    assert np.array_equal(gx, ref[1])                                           # grad_X does not depend on the update
+    assert np.array_equal(codes[1], ref[0][1]) and np.array_equal(codes[0][nh:], ref[0][0][nh:])
+    _, _, _, parts = O.fp8_step(case["chunks"], x, labels, 0.05, sr_mode="rtn", return_parts=True)
+    a = parts[0]["a"][:nh].astype(np.float64)
+    w0 = C.e4m3_decode(case["chunks"][0][:nh]).astype(np.float64)
+    exact = w0 + k0 - float(np.float32(0.05)) * a
+    got = C.e4m3_decode(codes[0][:nh]).astype(np.float64) + kn
+    assert np.abs(got - exact).max() <= 2.0 ** -8 * np.abs(kn).max() + 1e-7      # only the bf16 rounding of k' is lost
+    # reference offsets: sliced call for the rows behind the head
+    seeds = [77, 78]
+    c_sr, _, _, _ = O.fp8_kahan_step(case["chunks"], k0, x, labels, 0.05, nh, seeds=seeds, sr_mode="reference")
+    t_tail = parts[0]["t"][nh:]
+    offs = np.arange(64 - nh)[:, None] * 768 + np.arange(768)[None, :]
+    assert np.array_equal(c_sr[0][nh:], C.sr_e4m3_reference(t_tail, 77, offs))
+    # e5m2 buffer: same weights as long as the buffer values survive the coarser cast of the *previous* step (k0 = 0 here)
+    kz = np.zeros((nh, 768), dtype=np.uint8)
+    c8, k8, _, _ = O.fp8_kahan_step(case["chunks"], kz, x, labels, 0.05, nh, kahan_type="e5m2", sr_mode="rtn")
+    cb, kb, _, _ = O.fp8_kahan_step(case["chunks"], np.zeros((nh, 768), np.float32), x, labels, 0.05, nh, sr_mode="rtn")
+    assert np.array_equal(c8[0], cb[0]) and np.abs(C.e5m2_decode(k8) - kb).max() <= 2.0 ** -3 * np.abs(kb).max()

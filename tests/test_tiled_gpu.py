@@ -199,3 +199,92 @@ def test_fp8_module_simulated_mode(gpu):
         d = H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r)
         assert d.max() <= 1 and (d != 0).mean() < 2e-3
     assert xfc.grad_input.shape == (32, 768)
+
+
+def run_kahan(case, k0, ktype, nh, device, mode, seeds, lr=0.05):
+    import torch
+    from elmo_amd import ops
+    chunks, x, labels = H.to_device_case(case, device)
+    if ktype == "e5m2":
+        kt = torch.from_numpy(k0.copy()).to(device).view(torch.float8_e5m2)
+    else:
+        kt = torch.from_numpy(C.bf16_bits(k0).view(np.int16)).to(device).view(torch.bfloat16)
+    g, gf = ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", x, labels, lr, seeds=seeds, round_mode=mode, want_f32=True,
+                           quantize_x=True, saturate=True, kahan=kt, num_head=nh)
+    kn = kt.view(torch.uint8).cpu().numpy() if ktype == "e5m2" else kt.float().cpu().numpy()
+    return H.chunks_to_numpy(chunks), kn, gf.cpu().numpy(), g.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("ktype,mode", [("bf16", "rtn"), ("bf16", "sr_philox"), ("e5m2", "rtn")])
+def test_head_kahan_parity(gpu, ktype, mode):
+    """True-FP8 arithmetic on the three-kernel path with the compensated head (fuse_kernel.py:202-262)."""
+    case = H.make_case(2, 512, 32, 81)
+    nh = 208
+    rng = np.random.default_rng(2)
+    if ktype == "e5m2":
+        k0 = C.e5m2_encode(rng.standard_normal((nh, 768)).astype(np.float32) * 1e-3)
+    else:
+        k0 = C.bf16_round(rng.standard_normal((nh, 768)).astype(np.float32) * 1e-3)
+    seeds = [31337, 5] if mode != "rtn" else None
+    new, kn, gf, gb = run_kahan(case, k0, ktype, nh, gpu, mode, seeds)
+    ref_codes, ref_k, ref_gx, _ = O.fp8_kahan_step(case["chunks"], k0, case["x"], case["labels"], 0.05, nh, kahan_type=ktype,
+                                                   seeds=seeds, sr_mode="rtn" if mode == "rtn" else "reference")
+    mism = total = 0
+    for a, b in zip(new, ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1
+        mism += int((d != 0).sum()); total += d.size
+    assert mism / total < 2e-3
+    check_gx(gf, gb, ref_gx)
+    # the buffer: identical wherever the weight is (it holds what that rounding dropped); elsewhere it differs by the
+    # weight's grid step, so that weight + buffer still agree
+    same = new[0][:nh] == ref_codes[0][:nh]
+    kf = C.e5m2_decode(kn) if ktype == "e5m2" else kn
+    rf = C.e5m2_decode(ref_k) if ktype == "e5m2" else ref_k
+    tol = (2.0 ** -2 if ktype == "e5m2" else 2.0 ** -7) * np.abs(rf) + 1e-7
+    assert np.all(np.abs(kf - rf)[same] <= tol[same])
+    tot_g = C.e4m3_decode(new[0][:nh]).astype(np.float64) + kf
+    tot_r = C.e4m3_decode(ref_codes[0][:nh]).astype(np.float64) + rf
+    assert np.abs(tot_g - tot_r).max() <= (2.0 ** -2 if ktype == "e5m2" else 2.0 ** -6) * np.abs(rf).max() + 1e-6
+
+
+def test_true_fp8_on_the_tiled_path_matches_the_fused_oracle(gpu):
+    """quantize_x + saturate turn the three-kernel path into the arithmetic of the fused kernel (no buffer)."""
+    from elmo_amd import ops
+    case = H.make_case(2, 1024, 32, 82)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    g, gf = ops.tiled_step(chunks, 1024, "e4m3", x, labels, 0.05, round_mode="rtn", want_f32=True, quantize_x=True,
+                           saturate=True)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn")
+    for a, b in zip(H.chunks_to_numpy(chunks), ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx)
+
+
+def test_head_kahan_module(gpu):
+    import types
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked_head_kahan_fp8xmc_clf import Fp8XMCBCEChunkedHeadKahanLayer
+    cfg = make_cfg("cuda:0", 1000, 2, rounding="rtn")
+    cfg.training.FP8 = types.SimpleNamespace(using_head_kahan=True, fp8_head_kahan=False, head_ratio=0.2)
+    torch.manual_seed(0)
+    xfc = Fp8XMCBCEChunkedHeadKahanLayer(cfg)
+    assert xfc.num_labels == 1024 and xfc.num_head == 204 and xfc.head_kahan.shape == (204, 768)
+    assert xfc.head_kahan.dtype == torch.bfloat16 and sorted(xfc.state_dict().keys()) == ["xfc_weight.0", "xfc_weight.1"]
+    tokens = torch.randn(32, 768, device=gpu, dtype=torch.bfloat16) * 0.05
+    labels = torch.tensor([[0, 3], [31, 999], [4, 100]], dtype=torch.int32, device=gpu)
+    before = [w.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    assert xfc.xfc_forward_backward(tokens, labels, [0.05]) == 0 and xfc.iteration == 1
+    ref_codes, ref_k, _, _ = O.fp8_kahan_step(before, np.zeros((204, 768), np.float32), tokens.float().cpu().numpy(),
+                                              labels.cpu().numpy(), 0.05, 204, sr_mode="rtn")
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        d = H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r)
+        assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    assert float(xfc.head_kahan.float().abs().max()) > 0            # the buffer picked up the rounding residue
+    assert xfc.xfc_forward(tokens).shape == (32, 1000)
+    cfg2 = make_cfg("cuda:0", 1000, 2)
+    cfg2.training.FP8 = types.SimpleNamespace(using_head_kahan=False, fp8_head_kahan=False, head_ratio=0.2)
+    plain = Fp8XMCBCEChunkedHeadKahanLayer(cfg2)                      # no buffer: the fused kernel
+    assert plain.xfc_forward_backward(tokens, labels, [0.05]) == 0 and not hasattr(plain, "head_kahan")
