@@ -24,9 +24,10 @@
 //               grad_X[64h.. x 48fg..] += G^T W_t   v_mfma_f32_16x16x32_bf16, W via ds_read_b64_tr_b8 + fp8->bf16
 //               A^T[48fg.. x 32h..]     = X^T G^T    v_mfma_f32_16x16x32_bf16, G via ds_read_b64_tr_b16
 //               W_t = round(W - lr A) from registers to memory, 12 bytes per lane and row
-// All loads of an iteration are issued right after its barrier and consumed after the next one.  Tile descriptors
-// and the counters come in through LDS as well (a "mailbox"), so that no load result is ever waited for in
-// registers and the only memory wait of the loop is the one in front of the barrier.
+// Loads are direct-to-LDS, issued one at a time between the compute phases and consumed two iterations later: the
+// wait in front of the per-tile barrier leaves the operations of the iteration just finished in flight, so neither
+// the issue nor the latency of a load is waited for.  Tile descriptors come through the scalar path (they are
+// constant during the launch); a snapshot of the counters arrives in LDS with the other loads.
 // A member may overwrite its columns of tile t only after every member has published G(t), i.e. has finished
 // reading the rows of tile t; the counters guarantee it.  All waits on counters are bounded and raise an
 // error word instead of hanging.
@@ -41,20 +42,20 @@ constexpr int QNT = 512;                  // threads per workgroup (8 wavefronts
 constexpr int QCOLS = D / 4;              // features owned by one member (192)
 constexpr int QWS = QCOLS + 16;           // LDS row stride of the own-column tile image (13 x 16 bytes)
 constexpr int QWC_BYTES = TL * QWS;       // 13312
-constexpr int QRING = 6;                  // own-column tile images in flight
+constexpr int QRING = 3;                  // own-column tile images: in use, landed, in flight
 constexpr int QPL_S = TL * 2 + 16;        // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
 constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432 = 18 wave-wide loads), padded
-constexpr int QSLOTS = 8;                 // exchange slots per quad
+constexpr int QSLOTS = 16;                // exchange slots per quad
 constexpr int QLDS_G = QRING * QWC_BYTES; // LDS offset of the two gathered-G buffers
 constexpr int QRS = D + 16;               // LDS row stride of the own-rows image (49 x 16 bytes)
 constexpr int QROW_BYTES = 13 * 1024;     // 16 rows x 784 = 12544, padded to 13 wave-wide loads
 constexpr int QRRING = 3;                 // own-rows images in flight
-constexpr int QLDS_R = QLDS_G + 2 * QG_BYTES;
-constexpr int QLDS_M = QLDS_R + QRRING * QROW_BYTES;   // two mailboxes of 256 bytes
-constexpr int QLDS_BYTES = QLDS_M + 2 * 256;
+constexpr int QGBUF = 3;                  // gathered-G buffers: in use, landed, in flight
+constexpr int QLDS_R = QLDS_G + QGBUF * QG_BYTES;
+constexpr int QLDS_M = QLDS_R + QRRING * QROW_BYTES;   // four snapshots of the counters, 16 bytes each
+constexpr int QLDS_BYTES = QLDS_M + 256;
 constexpr int QSPIN_LIMIT = 1 << 18;
-constexpr int QAHEAD = 4;                 // stage A runs this many tiles ahead of stage B
-constexpr int QINF = QAHEAD + 3;          // tile descriptors held in scalar registers
+constexpr int QAHEAD = 7;                 // stage A runs this many tiles ahead of stage B
 
 struct QuadParams {
   unsigned char* chunk[MAX_CHUNKS];   // device pointers of the chunk weight tensors [rows_per_chunk, 768] e4m3
@@ -96,6 +97,11 @@ __device__ __forceinline__ void q_lds_load16(const unsigned char* g, unsigned ld
   const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsoff), "v"(g) : "memory", "m0");
 }
+// same with a wave-uniform base pointer and a 32-bit per-lane byte offset
+__device__ __forceinline__ void q_lds_load16_sbase(const unsigned char* base, unsigned off, unsigned ldsoff_) {
+  const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsoff), "v"(off), "s"(base) : "memory", "m0");
+}
 // same, at device scope (sc1): never served by this compute unit's L1, which may still hold the previous contents
 // of an exchange slot
 __device__ __forceinline__ void q_lds_load16_l2(const unsigned char* g, unsigned ldsoff_) {
@@ -116,19 +122,30 @@ __device__ __forceinline__ bf16x8 q_fp8x8_to_bf16x8(intx2 raw) {
 }
 
 // Everything the kernel needs to know about one tile; wave-uniform, kept in scalar registers.  The descriptors are
-// precomputed by tile_desc_kernel.
+// precomputed by quad_desc_prep_kernel (32 bytes: {base pointer, valid rows, seed}, {first key, one past the last key,
+// row in chunk, first label}) and read through the scalar (constant) path: they do not change during the launch.
 struct QTile { unsigned char* base; unsigned label0; int row0, rows_valid, p0, p1; unsigned seed; };
+typedef const __attribute__((address_space(4))) intx4 q_cdesc;
 
-__device__ __forceinline__ QTile q_from_desc(uint4 d0, uint4 d1) {
-  QTile q;
-  const unsigned lo = __builtin_amdgcn_readfirstlane(d0.x), hi = __builtin_amdgcn_readfirstlane(d0.y);
-  q.base = (unsigned char*)(((unsigned long long)hi << 32) | lo);
-  q.seed = __builtin_amdgcn_readfirstlane(d0.z);
-  q.p0 = (int)__builtin_amdgcn_readfirstlane(d0.w);
-  q.p1 = (int)__builtin_amdgcn_readfirstlane(d1.x);
-  q.row0 = (int)__builtin_amdgcn_readfirstlane(d1.y);
-  q.rows_valid = (int)__builtin_amdgcn_readfirstlane(d1.z);
-  q.label0 = __builtin_amdgcn_readfirstlane(d1.w);
+// base pointer and valid rows only
+__device__ __forceinline__ q_cdesc* q_desc_ptr(q_cdesc* desc, int t) {
+  return (q_cdesc*)((const __attribute__((address_space(4))) unsigned char*)desc + ((unsigned)t << 5));
+}
+__device__ __forceinline__ QTile q_desc_head(q_cdesc* desc, int t) {
+  const intx4 d0 = q_desc_ptr(desc, t)[0];
+  QTile q = {};
+  q.base = (unsigned char*)(((unsigned long long)(unsigned)d0.y << 32) | (unsigned)d0.x);
+  q.rows_valid = d0.z;
+  q.seed = (unsigned)d0.w;
+  return q;
+}
+__device__ __forceinline__ QTile q_desc_full(q_cdesc* desc, int t) {
+  QTile q = q_desc_head(desc, t);
+  const intx4 d1 = q_desc_ptr(desc, t)[1];
+  q.p0 = d1.x;
+  q.p1 = d1.y;
+  q.row0 = d1.z;
+  q.label0 = (unsigned)d1.w;
   return q;
 }
 
@@ -180,7 +197,7 @@ __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* 
                                                    unsigned short* xt);
 
 // Second launch: blocks below desc_blocks write, for every tile,
-//   desc[t] = {base pointer, seed, first key | one past last key, row in chunk, valid rows, first label}
+//   desc[t] = {base pointer, valid rows, seed | first key, one past the last key, row in chunk, first label}
 //   tile_ptr[t] = first key whose label >= first label of tile t (binary search in the sorted keys)
 // and the remaining blocks build the operand images of X.
 __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p, int n_pad, int* tile_ptr, uint4* desc, int desc_blocks,
@@ -209,9 +226,8 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
     const int c = t / p.tiles_per_chunk;
     const int row0 = (t - c * p.tiles_per_chunk) * TL;
     const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
-    desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), p.seed[c], (unsigned)p0};
-    desc[2 * t + 1] = uint4{(unsigned)p1, (unsigned)row0, (unsigned)min(TL, p.rows_per_chunk - row0),
-                            (unsigned)(c * p.rows_per_chunk + row0)};
+    desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), (unsigned)min(TL, p.rows_per_chunk - row0), p.seed[c]};
+    desc[2 * t + 1] = uint4{(unsigned)p0, (unsigned)p1, (unsigned)row0, (unsigned)(c * p.rows_per_chunk + row0)};
   }
 }
 
@@ -251,87 +267,84 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     for (int b = 0; b < 3; b++) acc2[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   QT_DECL
-  // own-column tile image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 wave-wide loads
-  auto issue_wcol = [&](int i, const QTile& q) {
-    if (i >= n_it) return;
-    const unsigned dst = (unsigned)((i % QRING) * QWC_BYTES);
+  // Per-lane source rows and byte offsets of the wave-wide pieces this wavefront loads (pieces v and v+8 of an image).
+  // own-column image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 pieces of 1 KiB
+  // own-rows image:   rows 16m..16m+15, 16 x 49 chunks of 16 bytes (48 data + 1 pad) = 13 pieces
+  int wrow[2], wcol_off[2], rrow[2], rcol_off[2];
 #pragma unroll
-    for (int s = 0; s < 2; s++) {
-      const int piece = v + 8 * s;
-      if (piece < 13) {
-        int ch = piece * 64 + lane;
-        int row = ch / 13, cc = ch - row * 13;
-        row = min(row, q.rows_valid - 1);
-        cc = min(cc, 11);
-        q_lds_load16(q.base + (size_t)row * D + QCOLS * m + cc * 16, dst + piece * 1024);
-      }
-    }
+  for (int s = 0; s < 2; s++) {
+    const int ch = (v + 8 * s) * 64 + lane;
+    wrow[s] = ch / 13;
+    wcol_off[s] = QCOLS * m + min(ch - wrow[s] * 13, 11) * 16;
+    const int rr = ch / 49;
+    rrow[s] = 16 * m + min(rr, 15);
+    rcol_off[s] = min(ch - rr * 49, 47) * 16;
+  }
+  q_cdesc* cdesc = (q_cdesc*)p.desc;
+  // tile index of position k in this quad's sequence; positions past the end fall back to tile 0, whose data is
+  // loaded and never used
+  auto tile_at = [&](int k) { const int t = quad + nquads * k; return t < p.num_tiles ? t : 0; };
+  auto wcol_piece = [&](int slot, const QTile& q, int s) {
+    if (v + 8 * s >= 13) return;
+    const unsigned off = (unsigned)(min(wrow[s], q.rows_valid - 1) * D + wcol_off[s]);
+    q_lds_load16_sbase(q.base, off, (unsigned)(slot * QWC_BYTES + (v + 8 * s) * 1024));
   };
-  // own-rows image: rows 16m..16m+15 of tile i, 16 x 49 chunks of 16 bytes (48 data + 1 pad) = 13 wave-wide loads
-  auto issue_rows = [&](int i, const QTile& q) {
-    if (i >= n_it) return;
-    const unsigned dst = (unsigned)(QLDS_R + (i % QRRING) * QROW_BYTES);
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-      const int piece = v + 8 * s;
-      if (piece < 13) {
-        int ch = piece * 64 + lane;
-        int row = ch / 49, cc = ch - row * 49;
-        row = max(min(16 * m + min(row, 15), q.rows_valid - 1), 0);
-        cc = min(cc, 47);
-        q_lds_load16(q.base + (size_t)row * D + cc * 16, dst + piece * 1024);
-      }
-    }
+  auto rows_piece = [&](int slot, const QTile& q, int s) {
+    if (v + 8 * s >= 13) return;
+    const unsigned off = (unsigned)(min(rrow[s], q.rows_valid - 1) * D + rcol_off[s]);
+    q_lds_load16_sbase(q.base, off, (unsigned)(QLDS_R + slot * QROW_BYTES + (v + 8 * s) * 1024));
   };
-  // the G tile of tile i: 18 wave-wide loads of 1 KiB
-  auto issue_gather = [&](int i) {
-    if (i >= n_it) return;
-    const unsigned char* src = p.exch + ((size_t)(quad * QSLOTS + (i & (QSLOTS - 1)))) * QG_BYTES;
-    const unsigned dst = (unsigned)(QLDS_G + (i & 1) * QG_BYTES);
-#pragma unroll
-    for (int s = 0; s < 3; s++) {
-      const int piece = v + 8 * s;
-      if (piece < 18) q_lds_load16_l2(src + piece * 1024 + lane * 16, dst + piece * 1024);
-    }
+  // the G tile of position i: 18 pieces of 1 KiB (pieces v, v+8, v+16)
+  const unsigned char* gsrc_lane = p.exch + (size_t)quad * QSLOTS * QG_BYTES + v * 1024 + lane * 16;
+  auto gather_piece = [&](int i, int slot, int s) {
+    if (v + 8 * s >= 18) return;
+    q_lds_load16_l2(gsrc_lane + (i & (QSLOTS - 1)) * QG_BYTES + s * 8192, (unsigned)(QLDS_G + slot * QG_BYTES + (v + 8 * s) * 1024));
   };
-  // mailbox of iteration i (wavefront 0 only): the descriptor of tile i+QINF (8 dwords) and the four counters
+  // snapshot of the four counters of iteration i (wavefront 0 only), read two iterations later
   auto issue_mailbox = [&](int i) {
     if (v != 0) return;
-    const int t = quad + nquads * (i + QINF);
-    const unsigned* dsrc = (const unsigned*)(p.desc + 2 * (size_t)(t < p.num_tiles ? t : 0));
-    const void* src = lane < 8 ? (const void*)(dsrc + lane) : (const void*)(flags + (lane & 3));
-    q_lds_load4_l2(src, (unsigned)(QLDS_M + (i & 1) * 256));
+    if (lane < 4) q_lds_load4_l2(flags + lane, (unsigned)(QLDS_M + (i & 3) * 16));
   };
-  // stage A of tile i: logits of label rows 16m.. against batch rows 16v.., sigmoid minus target, store this
-  // wavefront's part of G to the exchange slot (published later, once the stores have completed)
-  auto stage_a = [&](int i, const QTile& q) {
-    if (i >= n_it) return;
+  auto lds_i4 = [&](unsigned off) { return *(const __attribute__((address_space(3))) intx4*)(lds + off); };
+  // stage A of the tile at position i: logits of label rows 16m.. against batch rows 16v.., sigmoid minus target, store
+  // this wavefront's part of G to the exchange slot (published later, once the stores have completed)
+  unsigned char* gdst_lane = p.exch + (size_t)quad * QSLOTS * QG_BYTES + (16 * v + l16) * QPL_S + (16 * m + 4 * kg) * 2;
+  auto stage_a = [&](int i, int slot, const QTile& q) {
     floatx4 z = floatx4{0.f, 0.f, 0.f, 0.f};
     {
       // lane (row l16, k group kg) holds 32 consecutive bytes per K step
-      const unsigned asrc = (unsigned)(QLDS_R + (i % QRRING) * QROW_BYTES) + l16 * QRS + kg * 32;
+      const unsigned asrc = (unsigned)(QLDS_R + slot * QROW_BYTES) + l16 * QRS + kg * 32;
+      // the reads of three K steps are in flight at a time
       intx4 alo[6], ahi[6];
-#pragma unroll
-      for (int ks = 0; ks < 6; ks++) {
+      auto rd = [&](int ks) {
         alo[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128);
         ahi[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128 + 16);
-      }
+      };
+      rd(0); rd(1); rd(2);
+      QFENCE();
 #pragma unroll
       for (int ks = 0; ks < 6; ks++) {
+        if (ks + 3 < 6) rd(ks + 3);
         intx8 av = intx8{alo[ks].x, alo[ks].y, alo[ks].z, alo[ks].w, ahi[ks].x, ahi[ks].y, ahi[ks].z, ahi[ks].w};
         z = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, xq[ks], z, 0, 0, 0, 0, 0, 0);
+        QFENCE();
       }
     }
     const float nlog2e = -1.44269504088896340736f;
     const int r0 = 16 * m + 4 * kg;   // this lane's label rows r0..r0+3; its batch row is 16v + l16
-    float sg[4];
+    // sigmoid of the bf16 logits, rounded to bf16 in pairs
+    unsigned zb[2], sb[2];
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      float zf = bf16_rt(z[e] * p.zscale);
-      sg[e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * nlog2e)));
+    for (int e2 = 0; e2 < 2; e2++) {
+      zb[e2] = bf16_pack2(z[2 * e2] * p.zscale, z[2 * e2 + 1] * p.zscale);
+      const float z0 = __uint_as_float(zb[e2] << 16), z1 = __uint_as_float(zb[e2] & 0xFFFF0000u);
+      sb[e2] = bf16_pack2(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z0 * nlog2e)),
+                          __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z1 * nlog2e)));
     }
     // positives of this tile (set semantics: a repeated key counts once); wave-uniform scalar loads
     if (q.p1 > q.p0) {
+      float sg[4] = {__uint_as_float(sb[0] << 16), __uint_as_float(sb[0] & 0xFFFF0000u), __uint_as_float(sb[1] << 16),
+                     __uint_as_float(sb[1] & 0xFFFF0000u)};
       for (int e = q.p0; e < q.p1; e++) {
         const unsigned key = ckeys[e];
         const unsigned prev = e > 0 ? ckeys[e - 1] : ~key;
@@ -341,15 +354,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         for (int q4 = 0; q4 < 4; q4++)
           if (mine && l == (unsigned)q4) sg[q4] = bf16_rt(sg[q4] - 1.0f);
       }
+      sb[0] = bf16_pack2(sg[0], sg[1]);
+      sb[1] = bf16_pack2(sg[2], sg[3]);
     }
-    unsigned char* dstp = p.exch + ((size_t)(quad * QSLOTS + (i & (QSLOTS - 1)))) * QG_BYTES + (16 * v + l16) * QPL_S + r0 * 2;
-    unsigned short sb[4];
+    if (q.rows_valid < TL) {   // rows past the end of the chunk contribute nothing
 #pragma unroll
-    for (int e = 0; e < 4; e++) sb[e] = (r0 + e < q.rows_valid) ? bf16_bits(sg[e]) : (unsigned short)0;
-    uint2 o;
-    o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
-    o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
-    *(uint2*)dstp = o;
+      for (int e2 = 0; e2 < 2; e2++) {
+        if (r0 + 2 * e2 >= q.rows_valid) sb[e2] &= 0xFFFF0000u;
+        if (r0 + 2 * e2 + 1 >= q.rows_valid) sb[e2] &= 0x0000FFFFu;
+      }
+    }
+    *(uint2*)(gdst_lane + (i & (QSLOTS - 1)) * QG_BYTES) = uint2{sb[0], sb[1]};
   };
   // wait until every member has published at least `need` tiles (fmin: the smallest counter seen earlier, which
   // normally suffices; the polling loop is kept out of the common path)
@@ -366,82 +381,91 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     }
   };
 
-  // ---- prologue: descriptors of the first QINF tiles, own columns of tiles 0..4, stage A of the first QAHEAD tiles,
-  //      own rows of the next two, gather of tile 0
-  QTile inf[QINF];     // inf[k] describes the tile k positions ahead of the current one
+  // ---- prologue: own columns and G of positions 0 and 1, stage A of the first QAHEAD positions, own rows of the
+  //      next two
 #pragma unroll
-  for (int k = 0; k < QINF; k++) {
-    const int t = quad + nquads * k;
-    const uint4* src = p.desc + 2 * (size_t)(t < p.num_tiles ? t : 0);
-    inf[k] = q_from_desc(src[0], src[1]);
+  for (int k = 0; k < 3; k++) {
+    const QTile t = q_desc_head(cdesc, tile_at(k));
+#pragma unroll
+    for (int s = 0; s < 2; s++) rows_piece(k, t, s);
   }
 #pragma unroll
-  for (int k = 0; k < 3; k++) issue_rows(k, inf[k]);
+  for (int k = 0; k < 2; k++) {
+    const QTile t = q_desc_head(cdesc, tile_at(k));
 #pragma unroll
-  for (int k = 0; k < 5; k++) issue_wcol(k, inf[k]);
+    for (int s = 0; s < 2; s++) wcol_piece(k, t, s);
+  }
 #pragma unroll
   for (int k = 0; k < QAHEAD; k++) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    stage_a(k, inf[k]);
+    if (k < n_it) stage_a(k, k % QRRING, q_desc_full(cdesc, tile_at(k)));
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (k + 3 < QAHEAD + 2) issue_rows(k + 3, inf[k + 3]);
+    if (k + 3 < QAHEAD + 2) {
+      const QTile t = q_desc_head(cdesc, tile_at(k + 3));
+#pragma unroll
+      for (int s = 0; s < 2; s++) rows_piece(k % QRRING, t, s);
+    }
   }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0 && n_it > 0) __hip_atomic_store(flags + m, min(QAHEAD, n_it), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (n_it > 0) wait_published(1, 0);
-  issue_gather(0);
-  int fmin = 0;
+  const int fboot = min(4, n_it);   // what the first two iterations need of the counters
+  if (n_it > 0) wait_published(fboot, 0);
+#pragma unroll
+  for (int k = 0; k < 2; k++)
+#pragma unroll
+    for (int s = 0; s < 3; s++) gather_piece(k, k, s);
 
-  bool prev_full = false;
+  // Vector memory operations retire in order.  A regular iteration issues a fixed number of them per wavefront, at
+  // least seven (pieces of G and of the own columns two positions ahead, of the own rows QAHEAD+2 positions ahead, the
+  // snapshot of the counters, its part of G of position i+QAHEAD and two stores of updated weights), spread over the
+  // iteration so that the memory pipeline accepts each at once.  The wait in front of the barrier leaves seven in
+  // flight: what iteration i consumes was issued in iteration i-2 or earlier, so neither the issue nor the latency
+  // of a load is ever waited for.  After an iteration that issued fewer (the last positions, a short tile)
+  // everything is waited for.  Loads for positions past the end fetch tile 0 into buffers nobody reads.
+  bool prev_regular = false;
+  int s0 = 0, s1 = 1, s2 = 2;   // i % 3, (i+1) % 3, (i+2) % 3
+  // descriptors of the next iteration: its tile, the tile of its stage A, the tiles whose rows and columns it fetches.
+  // They are loaded in front of the weight update of the iteration before, where their latency hides behind LDS reads.
+  QTile q_n = q_desc_full(cdesc, tile_at(0)), qa_n = q_desc_full(cdesc, tile_at(QAHEAD));
+  QTile qr_n = q_desc_head(cdesc, tile_at(QAHEAD + 2)), qw_n = q_desc_head(cdesc, tile_at(2));
   for (int i = 0; i < n_it; i++) {
-    // Vector memory operations retire in order.  The last two this wavefront issued in the previous iteration are
-    // its stores of updated weights; everything older - G of tile i, own columns and own rows of the tiles ahead,
-    // this member's G part of tile i+QAHEAD-1, the mailbox - was issued right after the previous barrier.  Leaving
-    // two operations in flight keeps the store latency off the critical path.  If the previous tile was not full,
-    // fewer stores were issued and the count could cover loads, so all are waited for.
-    if (prev_full) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+    if (prev_regular) asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     QT(0)
     __syncthreads();
     QT(1)
-    if (i > 0) {   // mailbox of the previous iteration: next descriptor and the counters
-      const unsigned mb_off = (unsigned)(QLDS_M + ((i - 1) & 1) * 256);
-      const intx4 r0 = *(const __attribute__((address_space(3))) intx4*)(lds + mb_off);
-      const intx4 r1 = *(const __attribute__((address_space(3))) intx4*)(lds + mb_off + 16);
-      const intx4 fl = *(const __attribute__((address_space(3))) intx4*)(lds + mb_off + 32);
-      const uint4 d0 = uint4{(unsigned)r0.x, (unsigned)r0.y, (unsigned)r0.z, (unsigned)r0.w};
-      const uint4 d1 = uint4{(unsigned)r1.x, (unsigned)r1.y, (unsigned)r1.z, (unsigned)r1.w};
-#pragma unroll
-      for (int k = 0; k + 1 < QINF; k++) inf[k] = inf[k + 1];
-      inf[QINF - 1] = q_from_desc(d0, d1);
+    const QTile q = q_n, qa = qa_n, qr = qr_n, qw = qw_n;
+    int fmin = fboot;
+    if (i >= 2) {   // the counters as they were two iterations ago
+      const intx4 fl = lds_i4((unsigned)(QLDS_M + ((i + 2) & 3) * 16));
       fmin = min(min((int)__builtin_amdgcn_readfirstlane(fl.x), (int)__builtin_amdgcn_readfirstlane(fl.y)),
                  min((int)__builtin_amdgcn_readfirstlane(fl.z), (int)__builtin_amdgcn_readfirstlane(fl.w)));
     }
-    const QTile q = inf[0];
-    const unsigned wc = (unsigned)((i % QRING) * QWC_BYTES);
-    const unsigned gb = (unsigned)(QLDS_G + (i & 1) * QG_BYTES);
-    prev_full = q.rows_valid == TL;
-    if (tid == 0 && i > 0 && i + QAHEAD - 1 < n_it)
-      __hip_atomic_store(flags + m, i + QAHEAD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-    // ---- all loads of this iteration: G of the next tile (published by every member at least one full iteration ago,
-    //      so the counters in the mailbox normally suffice), own rows six tiles ahead, own columns five tiles ahead,
-    //      the next mailbox
-    if (i + 1 < n_it) {
-      wait_published(i + 2, fmin);
-      issue_gather(i + 1);
-    }
-    issue_rows(i + QAHEAD + 2, inf[QAHEAD + 2]);
-    issue_wcol(i + 5, inf[5]);
-    issue_mailbox(i);
+    const unsigned wc = (unsigned)(s0 * QWC_BYTES);
+    const unsigned gb = (unsigned)(QLDS_G + s0 * QG_BYTES);
+    const bool do_a = i + QAHEAD < n_it;
+    prev_regular = q.rows_valid == TL && do_a;
+    // G of the positions up to i+QAHEAD-2 was stored in iteration i-2 or earlier: complete by the wait above
+    if (tid == 0 && i >= 2 && i + QAHEAD - 1 <= n_it)
+      __hip_atomic_store(flags + m, i + QAHEAD - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (i + 2 < n_it) wait_published(i + 3, fmin);
+    // the loads of this iteration, one at a time between the phases below
+    auto mem_piece = [&](int k) {
+      if (k < 3) gather_piece(i + 2, s2, k);
+      else if (k < 5) rows_piece(s0, qr, k - 3);
+      else if (k < 7) wcol_piece(s2, qw, k - 5);
+      else issue_mailbox(i);
+    };
+    mem_piece(0);
     QT(2)
 
     // The two wavefronts of a SIMD run stage A and grad_X in opposite orders, so that the LDS reads of one overlap
-    // the MFMAs of the other.  The stores of stage A stay ahead of the weight stores in both orders (see the wait above).
-    if (h == 0) stage_a(i + QAHEAD, inf[QAHEAD]);
+    // the MFMAs of the other.
+    if (h == 0 && do_a) stage_a(i + QAHEAD, s1, qa);
+    mem_piece(1);
     QT(3)
 
     // ---- grad_X[64 x 48] += G^T W; 6 steps (32-row K step major, 16-feature block minor); the transposed W read of
@@ -469,11 +493,16 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 #pragma unroll
         for (int mb = 0; mb < 4; mb++)
           acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[ks2][mb], wb[s & 1], acc2[mb][nn], 0, 0, 0);
+        mem_piece(2 + s);
       }
     }
-    if (h != 0) stage_a(i + QAHEAD, inf[QAHEAD]);
+    if (h != 0 && do_a) stage_a(i + QAHEAD, s1, qa);
     QT(4)
 
+    qa_n = q_desc_full(cdesc, tile_at(i + 1 + QAHEAD));
+    qr_n = q_desc_head(cdesc, tile_at(i + 1 + QAHEAD + 2));
+    qw_n = q_desc_head(cdesc, tile_at(i + 3));
+    q_n = q_desc_full(cdesc, tile_at(i + 1));
     // ---- A^T[48 features x 32 rows] = X^T G^T in two 16-row blocks, each followed by its update.  Row r = 4kg+e of
     //      feature block cg is feature 12kg + 4cg + e of the wavefront's 48, so that a lane ends up with 12
     //      consecutive bytes of one weight row.
@@ -522,8 +551,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       }
     }
     QT(5)
+    { const int t = s0; s0 = s1; s1 = s2; s2 = t; }
   }
 
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last descriptor fetches still target LDS
 #ifdef XMC_TIMING
   if (lane == 0 && g < 48)
     for (int k = 0; k < 8; k++) p.flags[1024 + (g * 8 + v) * 8 + k] = (int)tacc[k];
