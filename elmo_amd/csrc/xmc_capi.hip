@@ -29,8 +29,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
-    (void)hipFuncSetAttribute((const void*)sort_keys_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
-    (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_POS * 4);
+    (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
   }
   return cached[dev];
 }
@@ -120,12 +119,13 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
   const int num_tiles = num_chunks * tiles_per_chunk;
   int n_pad = 0;
-  if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
+  if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
   if (step_kernel_choice() == 1) {
     (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
     if (n_pad > 0)
-      sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS));
+      quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch,
+                                                                            (unsigned*)(ws + WS_KEYS), nullptr);
     tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
                                                                   tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
     prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
@@ -182,8 +182,8 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.batch = batch;
     const int qgrid = grid / 32 * 32;   // whole quads on every XCD
     if (qgrid < 32) return XMC_ERR_DEVICE;
-    quad_sort_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS),
-                                                            (int*)(ws + WS_FLAGS));
+    quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
+        labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
     quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, 0, stream>>>(
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
@@ -196,7 +196,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
-    reduce_gx_quad_kernel<<<48, QNT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+    reduce_gx_quad_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
                                                  (unsigned short*)grad_x_bf16, batch);
   }
   return launch_status();
@@ -277,10 +277,10 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   unsigned short* gbl = glb + (size_t)rows_pad * BP;
   int* tile_ptr = (int*)(gbl + (size_t)rows_pad * BP);
   int n_pad = 0;
-  if (nnz > 0) { n_pad = 1; while (n_pad < nnz) n_pad <<= 1; }
+  if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
   if (n_pad > 0)
-    sort_keys_kernel<<<1, 1024, (size_t)n_pad * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys);
+    quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys, nullptr);
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
   tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, quantize_x, xb, xT);
   tiled_zero_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>(gx_total, BP * D);

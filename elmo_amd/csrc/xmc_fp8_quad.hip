@@ -149,48 +149,47 @@ __device__ __forceinline__ QTile q_desc_full(q_cdesc* desc, int t) {
   return q;
 }
 
-// First of the two launches in front of the step kernel (single workgroup): clear the counters and sort the positives
-// (key = label*256 + batch row, invalid entries -> 0xFFFFFFFF).  Up to 2048 keys are sorted by rank - every thread counts
-// the keys that precede its own, one pass over LDS with no barriers in between - larger sets by a bitonic network.
-__global__ __launch_bounds__(1024) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys, int* flags) {
+// First of the two launches in front of the step kernel: clear the counters (flags, may be null) and sort the positives
+// (key = label*256 + batch row, invalid entries -> 0xFFFFFFFF) by rank.  Workgroup b ranks keys 64b..64b+63 of the n_pad
+// (a power of two, at least 64, or 0): every workgroup builds all keys in LDS, its four wavefronts each count the keys
+// that precede the workgroup's own over a quarter of the set (equal keys: the one that comes first in the input
+// precedes), and the sum of the four counts is the key's position in the output.  Grid: max(1, n_pad / 64) x 256
+// threads, (n_pad + 256) * 4 bytes of LDS.
+__global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys, int* flags) {
   extern __shared__ unsigned sk[];
-  const int tid = threadIdx.x;
-  flags[tid] = 0;
-  for (int i = tid; i < n_pad; i += 1024) {
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+  if (blockIdx.x == 0 && flags)
+    for (int i = tid; i < 1024; i += 256) flags[i] = 0;
+  if (n_pad == 0) return;
+  for (int i = tid; i < n_pad; i += 256) {
     unsigned key = 0xFFFFFFFFu;
     if (i < nnz) {
-      int r = coo[2 * i], l = coo[2 * i + 1];
-      if (r >= 0 && r < batch && l >= 0 && l < (1 << 24) - 1) key = ((unsigned)l << 8) | (unsigned)r;
+      int r = coo[2 * i], lab = coo[2 * i + 1];
+      if (r >= 0 && r < batch && lab >= 0 && lab < (1 << 24) - 1) key = ((unsigned)lab << 8) | (unsigned)r;
     }
     sk[i] = key;
   }
   __syncthreads();
-  if (n_pad <= 2048) {
-    for (int i = tid; i < n_pad; i += 1024) {
-      const unsigned mine = sk[i];
-      int rank = 0;
-      for (int j = 0; j < n_pad; j++) {
-        const unsigned o = sk[j];
-        rank += (o < mine || (o == mine && j < i)) ? 1 : 0;
-      }
-      keys[rank] = mine;
-    }
-    return;
-  }
-  for (int k = 2; k <= n_pad; k <<= 1) {
-    for (int jj = k >> 1; jj > 0; jj >>= 1) {
-      for (int i = tid; i < n_pad; i += 1024) {
-        int ixj = i ^ jj;
-        if (ixj > i) {
-          unsigned a = sk[i], b = sk[ixj];
-          bool up = (i & k) == 0;
-          if ((a > b) == up) { sk[i] = b; sk[ixj] = a; }
-        }
-      }
-      __syncthreads();
+  const int i0 = blockIdx.x * 64;
+  const unsigned mine = sk[i0 + l];
+  const int quarter = n_pad >> 2;
+  int rank = 0;
+  for (int j = w * quarter; j < (w + 1) * quarter; j += 4) {   // groups of four never straddle the own range
+    const unsigned o0 = sk[j], o1 = sk[j + 1], o2 = sk[j + 2], o3 = sk[j + 3];
+    if (j < i0) {
+      rank += (o0 <= mine) + (o1 <= mine) + (o2 <= mine) + (o3 <= mine);
+    } else if (j >= i0 + 64) {
+      rank += (o0 < mine) + (o1 < mine) + (o2 < mine) + (o3 < mine);
+    } else {
+      const int me = i0 + l;
+      rank += (o0 < mine || (o0 == mine && j < me)) + (o1 < mine || (o1 == mine && j + 1 < me)) +
+              (o2 < mine || (o2 == mine && j + 2 < me)) + (o3 < mine || (o3 == mine && j + 3 < me));
     }
   }
-  for (int i = tid; i < n_pad; i += 1024) keys[i] = sk[i];
+  unsigned* part = sk + n_pad;
+  part[tid] = (unsigned)rank;
+  __syncthreads();
+  if (w == 0) keys[part[l] + part[64 + l] + part[128 + l] + part[192 + l]] = mine;
 }
 
 __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
@@ -567,11 +566,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * QNT + tid] = acc2[mb][nn];
 }
 
-// grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768]
-__global__ __launch_bounds__(QNT) void reduce_gx_quad_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
+// grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768].  192 workgroups of 128
+// threads: workgroup (slot, m, part) covers threads 128 part.. of the step kernel's workgroup layout.
+__global__ __launch_bounds__(128) void reduce_gx_quad_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
                                                              unsigned short* gx_bf16, int batch) {
-  const int slot = blockIdx.x >> 2, m = blockIdx.x & 3;   // slot = mb*3+nn
-  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int slot = blockIdx.x >> 4, m = (blockIdx.x >> 2) & 3;   // slot = mb*3+nn
+  const int tid = (blockIdx.x & 3) * 128 + threadIdx.x, v = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fg = v & 3, h = v >> 2;
   // the workgroups of member m, in a fixed order; eight loads in flight at a time
   floatx4 s = {0.f, 0.f, 0.f, 0.f};

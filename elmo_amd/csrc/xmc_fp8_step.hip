@@ -405,35 +405,6 @@ __global__ void prep_x_kernel(const unsigned short* x, int batch, float inv_scal
   }
 }
 
-// Sort the positives of one step and drop nothing: key = label*256 + batch_row, invalid entries -> 0xFFFFFFFF.
-// Single workgroup, bitonic network in LDS (n_pad = power of two <= MAX_POS).
-__global__ __launch_bounds__(1024) void sort_keys_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys) {
-  extern __shared__ unsigned sk[];
-  for (int i = threadIdx.x; i < n_pad; i += blockDim.x) {
-    unsigned key = 0xFFFFFFFFu;
-    if (i < nnz) {
-      int r = coo[2 * i], l = coo[2 * i + 1];
-      if (r >= 0 && r < batch && l >= 0 && l < (1 << 24) - 1) key = ((unsigned)l << 8) | (unsigned)r;
-    }
-    sk[i] = key;
-  }
-  __syncthreads();
-  for (int k = 2; k <= n_pad; k <<= 1) {
-    for (int jj = k >> 1; jj > 0; jj >>= 1) {
-      for (int i = threadIdx.x; i < n_pad; i += blockDim.x) {
-        int ixj = i ^ jj;
-        if (ixj > i) {
-          unsigned a = sk[i], b = sk[ixj];
-          bool up = (i & k) == 0;
-          if ((a > b) == up) { sk[i] = b; sk[ixj] = a; }
-        }
-      }
-      __syncthreads();
-    }
-  }
-  for (int i = threadIdx.x; i < n_pad; i += blockDim.x) keys[i] = sk[i];
-}
-
 // tile_ptr[t] = first key whose label >= first label of tile t; tile_ptr[num_tiles] = first key past the last tile
 __global__ void tile_ptr_kernel(const unsigned* keys, int n_pad, int rows_per_chunk, int tiles_per_chunk, int num_tiles,
                                 int* tile_ptr) {
