@@ -37,8 +37,8 @@ constexpr size_t WS_XT = WS_XQ + (size_t)BP * D;              // bf16 grad_W ope
 constexpr size_t WS_KEYS = WS_XT + (size_t)BP * D * 2;        // sorted positive keys  MAX_POS*4
 constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // counters + error word (4 KiB), then 12 KiB of debug time stamps
 constexpr size_t WS_PARTIAL = WS_FLAGS + 16384;               // MAX_WG * 48 * 256 * 16 bytes of grad_X partials
-constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 48 * NT * 16;      // G exchange ring: 64 quads x 16 slots x 4 x 5 KiB
-constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 16 * 4 * 5120;  // tile_ptr[num_tiles + 1]
+constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 48 * NT * 16;      // G exchange ring: 64 quads x 8 slots x 4 x 5 KiB
+constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 8 * 4 * 5120;  // tile_ptr[num_tiles + 1]
 
 __device__ __forceinline__ float bf16_rt(float f) { return (float)(__bf16)f; }
 

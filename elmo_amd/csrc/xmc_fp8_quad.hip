@@ -42,20 +42,25 @@ constexpr int QNT = 512;                  // threads per workgroup (8 wavefronts
 constexpr int QCOLS = D / 4;              // features owned by one member (192)
 constexpr int QWS = QCOLS + 16;           // LDS row stride of the own-column tile image (13 x 16 bytes)
 constexpr int QWC_BYTES = TL * QWS;       // 13312
-constexpr int QRING = 3;                  // own-column tile images: in use, landed, in flight
-constexpr int QPL_S = TL * 2 + 16;        // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
-constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432 = 18 wave-wide loads), padded
-constexpr int QSLOTS = 16;                // exchange slots per quad
+constexpr int QRING = 6;                  // own-column tile images: in use, four landed or landing, one in flight
+#ifndef XMC_GPAD
+#define XMC_GPAD 16
+#endif
+constexpr int QPL_S = TL * 2 + XMC_GPAD;  // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
+constexpr int QG_PIECES = (BP * QPL_S + 1023) / 1024;   // wave-wide loads per G tile (18)
+constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432), padded
+constexpr int QSLOTS = 8;                 // exchange slots per quad
 constexpr int QLDS_G = QRING * QWC_BYTES; // LDS offset of the two gathered-G buffers
 constexpr int QRS = D + 16;               // LDS row stride of the own-rows image (49 x 16 bytes)
 constexpr int QROW_BYTES = 13 * 1024;     // 16 rows x 784 = 12544, padded to 13 wave-wide loads
 constexpr int QRRING = 3;                 // own-rows images in flight
-constexpr int QGBUF = 3;                  // gathered-G buffers: in use, landed, in flight
+constexpr int QGBUF = 2;                  // gathered-G buffers: in use, in flight
 constexpr int QLDS_R = QLDS_G + QGBUF * QG_BYTES;
 constexpr int QLDS_M = QLDS_R + QRRING * QROW_BYTES;   // four snapshots of the counters, 16 bytes each
 constexpr int QLDS_BYTES = QLDS_M + 256;
 constexpr int QSPIN_LIMIT = 1 << 18;
-constexpr int QAHEAD = 7;                 // stage A runs this many tiles ahead of stage B
+constexpr int QAHEAD = 5;                 // stage A runs this many tiles ahead of stage B
+constexpr int QWAHEAD = QRING - 1;        // own columns are fetched this many tiles ahead
 
 struct QuadParams {
   unsigned char* chunk[MAX_CHUNKS];   // device pointers of the chunk weight tensors [rows_per_chunk, 768] e4m3
@@ -296,13 +301,13 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   // the G tile of position i: 18 pieces of 1 KiB (pieces v, v+8, v+16)
   const unsigned char* gsrc_lane = p.exch + (size_t)quad * QSLOTS * QG_BYTES + v * 1024 + lane * 16;
   auto gather_piece = [&](int i, int slot, int s) {
-    if (v + 8 * s >= 18) return;
+    if (v + 8 * s >= QG_PIECES) return;
     q_lds_load16_l2(gsrc_lane + (i & (QSLOTS - 1)) * QG_BYTES + s * 8192, (unsigned)(QLDS_G + slot * QG_BYTES + (v + 8 * s) * 1024));
   };
-  // snapshot of the four counters of iteration i (wavefront 0 only), read two iterations later
+  // snapshot of the four counters of iteration i (wavefront 0 only), read in the next iteration
   auto issue_mailbox = [&](int i) {
     if (v != 0) return;
-    if (lane < 4) q_lds_load4_l2(flags + lane, (unsigned)(QLDS_M + (i & 3) * 16));
+    if (lane < 4) q_lds_load4_l2(flags + lane, (unsigned)(QLDS_M + (i & 1) * 16));
   };
   auto lds_i4 = [&](unsigned off) { return *(const __attribute__((address_space(3))) intx4*)(lds + off); };
   // stage A of the tile at position i: logits of label rows 16m.. against batch rows 16v.., sigmoid minus target, store
@@ -380,8 +385,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     }
   };
 
-  // ---- prologue: own columns and G of positions 0 and 1, stage A of the first QAHEAD positions, own rows of the
-  //      next two
+  // ---- prologue: own columns of the first QWAHEAD positions, stage A of the first QAHEAD positions, own rows of the
+  //      next two, G of position 0
 #pragma unroll
   for (int k = 0; k < 3; k++) {
     const QTile t = q_desc_head(cdesc, tile_at(k));
@@ -389,7 +394,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     for (int s = 0; s < 2; s++) rows_piece(k, t, s);
   }
 #pragma unroll
-  for (int k = 0; k < 2; k++) {
+  for (int k = 0; k < QWAHEAD; k++) {
     const QTile t = q_desc_head(cdesc, tile_at(k));
 #pragma unroll
     for (int s = 0; s < 2; s++) wcol_piece(k, t, s);
@@ -410,60 +415,64 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0 && n_it > 0) __hip_atomic_store(flags + m, min(QAHEAD, n_it), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const int fboot = min(4, n_it);   // what the first two iterations need of the counters
+  const int fboot = min(2, n_it);   // what the first iteration needs of the counters
   if (n_it > 0) wait_published(fboot, 0);
 #pragma unroll
-  for (int k = 0; k < 2; k++)
-#pragma unroll
-    for (int s = 0; s < 3; s++) gather_piece(k, k, s);
+  for (int s = 0; s < 3; s++) gather_piece(0, 0, s);
 
-  // Vector memory operations retire in order.  A regular iteration issues a fixed number of them per wavefront, at
-  // least seven (pieces of G and of the own columns two positions ahead, of the own rows QAHEAD+2 positions ahead, the
-  // snapshot of the counters, its part of G of position i+QAHEAD and two stores of updated weights), spread over the
-  // iteration so that the memory pipeline accepts each at once.  The wait in front of the barrier leaves seven in
-  // flight: what iteration i consumes was issued in iteration i-2 or earlier, so neither the issue nor the latency
-  // of a load is ever waited for.  After an iteration that issued fewer (the last positions, a short tile)
+  // Vector memory operations retire in order.  In a regular iteration every wavefront issues, in this order: the
+  // snapshot of the counters (wavefront 0), its pieces of G of the next position, its pieces of the own rows QAHEAD+2
+  // and of the own columns QWAHEAD positions ahead, and - somewhere behind the first piece of G - its part of G of
+  // position i+QAHEAD and two stores of updated weights.  The loads are spread over the iteration so that the memory
+  // pipeline accepts each at once.  The wait in front of the barrier leaves the last four operations in flight: the
+  // snapshot and G, which the next iteration consumes, have landed; rows, columns and stores are not needed before
+  // the iteration after.  A tile's rows and columns are fetched two iterations apart, so that the second fetch finds
+  // the tile in the XCD's L2.  After an iteration that issued fewer operations (the last positions, a short tile)
   // everything is waited for.  Loads for positions past the end fetch tile 0 into buffers nobody reads.
   bool prev_regular = false;
   int s0 = 0, s1 = 1, s2 = 2;   // i % 3, (i+1) % 3, (i+2) % 3
+  int w0 = 0;                   // i % QRING
   // descriptors of the next iteration: its tile, the tile of its stage A, the tiles whose rows and columns it fetches.
   // They are loaded in front of the weight update of the iteration before, where their latency hides behind LDS reads.
   QTile q_n = q_desc_full(cdesc, tile_at(0)), qa_n = q_desc_full(cdesc, tile_at(QAHEAD));
-  QTile qr_n = q_desc_head(cdesc, tile_at(QAHEAD + 2)), qw_n = q_desc_head(cdesc, tile_at(2));
+  QTile qr_n = q_desc_head(cdesc, tile_at(QAHEAD + 2)), qw_n = q_desc_head(cdesc, tile_at(QWAHEAD));
   for (int i = 0; i < n_it; i++) {
-    if (prev_regular) asm volatile("s_waitcnt vmcnt(7) lgkmcnt(0)" ::: "memory");
+    if (prev_regular) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     QT(0)
     __syncthreads();
     QT(1)
     const QTile q = q_n, qa = qa_n, qr = qr_n, qw = qw_n;
     int fmin = fboot;
-    if (i >= 2) {   // the counters as they were two iterations ago
-      const intx4 fl = lds_i4((unsigned)(QLDS_M + ((i + 2) & 3) * 16));
+    if (i >= 1) {   // the counters as they were one iteration ago
+      const intx4 fl = lds_i4((unsigned)(QLDS_M + ((i + 1) & 1) * 16));
       fmin = min(min((int)__builtin_amdgcn_readfirstlane(fl.x), (int)__builtin_amdgcn_readfirstlane(fl.y)),
                  min((int)__builtin_amdgcn_readfirstlane(fl.z), (int)__builtin_amdgcn_readfirstlane(fl.w)));
     }
-    const unsigned wc = (unsigned)(s0 * QWC_BYTES);
-    const unsigned gb = (unsigned)(QLDS_G + s0 * QG_BYTES);
+    const int sl[3] = {s0, s1, s2};
+    const int slot_rows = sl[(QAHEAD + 2) % 3], slot_a = sl[QAHEAD % 3];
+    const int slot_wcol = w0 == 0 ? QRING - 1 : w0 - 1;   // (i + QWAHEAD) % QRING
+    const unsigned wc = (unsigned)(w0 * QWC_BYTES);
+    const unsigned gb = (unsigned)(QLDS_G + (i & 1) * QG_BYTES);
     const bool do_a = i + QAHEAD < n_it;
     prev_regular = q.rows_valid == TL && do_a;
     // G of the positions up to i+QAHEAD-2 was stored in iteration i-2 or earlier: complete by the wait above
     if (tid == 0 && i >= 2 && i + QAHEAD - 1 <= n_it)
       __hip_atomic_store(flags + m, i + QAHEAD - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (i + 2 < n_it) wait_published(i + 3, fmin);
+    issue_mailbox(i);
+    if (i + 1 < n_it) wait_published(i + 2, fmin);
     // the loads of this iteration, one at a time between the phases below
     auto mem_piece = [&](int k) {
-      if (k < 3) gather_piece(i + 2, s2, k);
-      else if (k < 5) rows_piece(s0, qr, k - 3);
-      else if (k < 7) wcol_piece(s2, qw, k - 5);
-      else issue_mailbox(i);
+      if (k < 3) gather_piece(i + 1, (i + 1) & 1, k);
+      else if (k < 5) rows_piece(slot_rows, qr, k - 3);
+      else if (k < 7) wcol_piece(slot_wcol, qw, k - 5);
     };
     mem_piece(0);
     QT(2)
 
     // The two wavefronts of a SIMD run stage A and grad_X in opposite orders, so that the LDS reads of one overlap
     // the MFMAs of the other.
-    if (h == 0 && do_a) stage_a(i + QAHEAD, s1, qa);
+    if (h == 0 && do_a) stage_a(i + QAHEAD, slot_a, qa);
     mem_piece(1);
     QT(3)
 
@@ -495,12 +504,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         mem_piece(2 + s);
       }
     }
-    if (h != 0 && do_a) stage_a(i + QAHEAD, s1, qa);
+    if (h != 0 && do_a) stage_a(i + QAHEAD, slot_a, qa);
     QT(4)
 
     qa_n = q_desc_full(cdesc, tile_at(i + 1 + QAHEAD));
     qr_n = q_desc_head(cdesc, tile_at(i + 1 + QAHEAD + 2));
-    qw_n = q_desc_head(cdesc, tile_at(i + 3));
+    qw_n = q_desc_head(cdesc, tile_at(i + 1 + QWAHEAD));
     q_n = q_desc_full(cdesc, tile_at(i + 1));
     // ---- A^T[48 features x 32 rows] = X^T G^T in two 16-row blocks, each followed by its update.  Row r = 4kg+e of
     //      feature block cg is feature 12kg + 4cg + e of the wavefront's 48, so that a lane ends up with 12
@@ -551,6 +560,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     }
     QT(5)
     { const int t = s0; s0 = s1; s1 = s2; s2 = t; }
+    w0 = w0 == QRING - 1 ? 0 : w0 + 1;
   }
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last descriptor fetches still target LDS
