@@ -421,12 +421,13 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   for (int s = 0; s < 3; s++) gather_piece(0, 0, s);
 
   // Vector memory operations retire in order.  In a regular iteration every wavefront issues, in this order: the
-  // snapshot of the counters (wavefront 0), its pieces of G of the next position, its pieces of the own rows QAHEAD+2
-  // and of the own columns QWAHEAD positions ahead, and - somewhere behind the first piece of G - its part of G of
-  // position i+QAHEAD and two stores of updated weights.  The loads are spread over the iteration so that the memory
-  // pipeline accepts each at once.  The wait in front of the barrier leaves the last four operations in flight: the
-  // snapshot and G, which the next iteration consumes, have landed; rows, columns and stores are not needed before
-  // the iteration after.  A tile's rows and columns are fetched two iterations apart, so that the second fetch finds
+  // snapshot of the counters (wavefront 0), its pieces of G of the next position, its pieces of the own columns
+  // QWAHEAD and of the own rows QAHEAD+2 positions ahead, and two stores of updated weights; its part of G of position
+  // i+QAHEAD is stored behind the first piece of G (h = 0) or behind the rows (h = 1).  The loads are spread over the
+  // iteration so that the memory pipeline accepts each at once.  The wait in front of the barrier leaves the last four
+  // (h = 0) or five (h = 1) operations in flight, which always include the rows - the only loads that miss the L2:
+  // the snapshot and G, which the next iteration consumes, have landed; rows, columns and stores are not needed
+  // before the iteration after.  A tile's rows and columns are fetched two iterations apart, so that the second fetch finds
   // the tile in the XCD's L2.  After an iteration that issued fewer operations (the last positions, a short tile)
   // everything is waited for.  Loads for positions past the end fetch tile 0 into buffers nobody reads.
   bool prev_regular = false;
@@ -437,8 +438,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   QTile q_n = q_desc_full(cdesc, tile_at(0)), qa_n = q_desc_full(cdesc, tile_at(QAHEAD));
   QTile qr_n = q_desc_head(cdesc, tile_at(QAHEAD + 2)), qw_n = q_desc_head(cdesc, tile_at(QWAHEAD));
   for (int i = 0; i < n_it; i++) {
-    if (prev_regular) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    if (!prev_regular) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else if (h == 0) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
     QT(0)
     __syncthreads();
     QT(1)
@@ -464,8 +466,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     // the loads of this iteration, one at a time between the phases below
     auto mem_piece = [&](int k) {
       if (k < 3) gather_piece(i + 1, (i + 1) & 1, k);
-      else if (k < 5) rows_piece(slot_rows, qr, k - 3);
-      else if (k < 7) wcol_piece(slot_wcol, qw, k - 5);
+      else if (k < 5) wcol_piece(slot_wcol, qw, k - 3);
+      else if (k < 7) rows_piece(slot_rows, qr, k - 5);
     };
     mem_piece(0);
     QT(2)
