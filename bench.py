@@ -238,11 +238,12 @@ def main():
     algo_flops = 6.0 * cfg.batch * cfg.num_labels * cfg.dim
     t_roof = max(algo_flops / (FP8_PEAK_TFLOPS * 1e12), algo_bytes / (HBM_PEAK_GBS * 1e9))
     achieved_gbs = algo_bytes / (kernel_ms * 1e-3) / 1e9
+    kernel_name = "fp8_step_kernel" if os.environ.get("XMC_KERNEL") == "pair" else "fp8_step_quad_kernel"
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(f"{cfg.name}:{args.round}")
+            traffic = json.load(f).get(f"{kernel_name}:{cfg.name}:{args.round}")
 
     out = {
         "metric": "XMC classifier train steps/sec at 670K labels FP8",
@@ -254,7 +255,7 @@ def main():
                    "lr": cfg.lr, "rounding": args.round, "seed": cfg.seed},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "fp8_step_kernel" if os.environ.get("XMC_KERNEL") == "pair" else "fp8_step_quad_kernel",
+                     "kernel": kernel_name,
                      "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_flops_per_launch": algo_flops},
         "roofline_step_frac": t_roof / (ms_per_step * 1e-3),
