@@ -41,7 +41,7 @@ def load():
     lib.xmc_tiled_workspace_bytes.argtypes = [i32, i32]
     lib.xmc_tiled_step.restype = i32
     lib.xmc_tiled_step.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32, vp, i32, i32, vp, i32, f32,
-                                   ctypes.POINTER(ctypes.c_uint32), i32, i32, i32, vp, i32, i32, vp, vp, vp, sz, vp]
+                                   ctypes.POINTER(ctypes.c_uint32), i32, i32, i32, vp, i32, i32, vp, vp, vp, vp, sz, vp]
     lib.xmc_select_step_kernel.restype = i32
     lib.xmc_select_step_kernel.argtypes = [i32]
     lib.xmc_copy_probe.restype = i32

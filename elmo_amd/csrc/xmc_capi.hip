@@ -235,14 +235,15 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk) {
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
-  return TW_G + 2 * rows_pad * BP * 2 + ((tiles + 1) * 4 + 255) / 256 * 256;
+  // G in both orientations, tile_ptr (padded to 64 entries), one loss share per tile
+  return TW_G + 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 4 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
                    const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
                    const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
-                   int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes,
-                   void* stream_) {
+                   int num_head, void* grad_x_bf16, float* grad_x_f32, float* loss_out, void* workspace,
+                   size_t workspace_bytes, void* stream_) {
   if (!chunk_ptrs || !x_bf16 || !workspace || !grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
   if (kahan_type < 0 || kahan_type > 2 || (kahan_type != 0 && (weight_type != W_E4M3 || !kahan))) return XMC_ERR_MODE;
   if (kahan_type != 0 && (num_head < 0 || num_head > rows_per_chunk || !aligned16(kahan))) return XMC_ERR_SHAPE;
@@ -276,6 +277,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   unsigned short* glb = (unsigned short*)(ws + TW_G);
   unsigned short* gbl = glb + (size_t)rows_pad * BP;
   int* tile_ptr = (int*)(gbl + (size_t)rows_pad * BP);
+  float* loss_part = (float*)(tile_ptr + (num_tiles + 1 + 63) / 64 * 64);   // one share per tile
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
@@ -284,6 +286,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
   tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, quantize_x, xb, xT);
   tiled_zero_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>(gx_total, BP * D);
+  if (loss_out) tiled_zero_kernel<<<(num_tiles + 255) / 256, 256, 0, stream>>>(loss_part, num_tiles);
   for (int c = 0; c < num_chunks; c++) {
     void* w = chunk_ptrs[c];
     const int rows = c == num_chunks - 1 ? rows_last_chunk : rows_per_chunk;
@@ -295,11 +298,15 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     int range = (rp + T_SPLITS - 1) / T_SPLITS;
     range = (range + TL - 1) / TL * TL;
     const int splits = (rp + range - 1) / range;
+    const int* tp = tile_ptr + c * tiles_per_chunk;
+    float* lp = loss_part + c * tiles_per_chunk;
     if (weight_type == W_BF16) {
-      tiled_logits_kernel<W_BF16><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tile_ptr + c * tiles_per_chunk, label0, glb, gbl);
+      if (loss_out) tiled_logits_kernel<W_BF16, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
+      else tiled_logits_kernel<W_BF16, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
       tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
     } else {
-      tiled_logits_kernel<W_E4M3><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tile_ptr + c * tiles_per_chunk, label0, glb, gbl);
+      if (loss_out) tiled_logits_kernel<W_E4M3, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
+      else tiled_logits_kernel<W_E4M3, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
       tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
     }
     tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total);
@@ -312,6 +319,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     }
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
+  if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, num_tiles, loss_out);
   return launch_status();
 }
 

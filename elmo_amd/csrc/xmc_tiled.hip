@@ -64,10 +64,14 @@ __global__ void tiled_zero_kernel(float* p, int n) {
 
 // ---- logits, sigmoid minus targets.  One workgroup per 64 label rows, wavefront w takes rows 16w..16w+15 against the
 //      whole (padded) batch.  Writes G[l][b] and G^T[b][l]; rows beyond the chunk are written as zeros.
-template <int WT>
+//      LOSS: also the workgroup's share of the summed binary cross entropy of the bf16 logits z against the targets,
+//      sum over labels and batch rows of max(z, 0) - [positive] z + log(1 + exp(-|z|)), the quantity that
+//      _compute_loss of the reference is written to return (chunked.py:57-72), in fp32 and stored per workgroup for a
+//      fixed-order sum.
+template <int WT, bool LOSS>
 __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int rows, int rows_pad, const unsigned short* xb,
                                                            const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
-                                                           unsigned short* glb, unsigned short* gbl) {
+                                                           unsigned short* glb, unsigned short* gbl, int batch, float* loss_part) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int r0 = blockIdx.x * TL + 16 * wv;
   const int lrow = min(r0 + l16, rows - 1);
@@ -86,12 +90,19 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
   // acc[nb][e] = Z[label r0 + 4kg + e][batch 16nb + l16]
   const float nlog2e = -1.44269504088896340736f;
   float sg[8][4];
+  float lsum = 0.f;
 #pragma unroll
   for (int nb = 0; nb < 8; nb++)
 #pragma unroll
     for (int e = 0; e < 4; e++) {
       float zf = bf16_rt(acc[nb][e]);
-      sg[nb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * nlog2e)));
+      const float ex = __builtin_amdgcn_exp2f(zf * nlog2e);   // exp(-z)
+      sg[nb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + ex));
+      if (LOSS) {
+        acc[nb][e] = zf;   // kept for the positives below
+        if (r0 + 4 * kg + e < rows && 16 * nb + l16 < batch)
+          lsum += __builtin_fmaxf(zf, 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf) * 1.44269504088896340736f));
+      }
     }
   // positives of this tile (set semantics: a repeated key counts once)
   const int p0 = tile_ptr[blockIdx.x], p1 = tile_ptr[blockIdx.x + 1];
@@ -106,8 +117,20 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
       for (int nb = 0; nb < 8; nb++)
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++)
-          if ((b >> 4) == (unsigned)nb && l == (unsigned)q4) sg[nb][q4] = bf16_rt(sg[nb][q4] - 1.0f);
+          if ((b >> 4) == (unsigned)nb && l == (unsigned)q4) {
+            sg[nb][q4] = bf16_rt(sg[nb][q4] - 1.0f);
+            if (LOSS && r0 + 4 * kg + q4 < rows) lsum -= acc[nb][q4];
+          }
     }
+  }
+  if (LOSS) {
+    // lanes of a wavefront, then the four wavefronts, in a fixed order
+    __shared__ float wsum[4];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
+    if (lane == 0) wsum[wv] = lsum;
+    __syncthreads();
+    if (tid == 0) loss_part[blockIdx.x] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
   }
 #pragma unroll
   for (int nb = 0; nb < 8; nb++) {
@@ -122,6 +145,20 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
 #pragma unroll
     for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
   }
+}
+
+// sum of the per-workgroup loss shares in a fixed order (double precision), one workgroup
+__global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part, int n, float* loss_out) {
+  __shared__ double sh[256];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256) s += (double)loss_part[i];
+  sh[threadIdx.x] = s;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) sh[threadIdx.x] += sh[threadIdx.x + off];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *loss_out = (float)sh[0];
 }
 
 // ---- grad_X partial of one label range: C[128 x 192] = G^T[128 x R] W[R x 192].  blockIdx = fb + 4*split; wavefront w

@@ -108,14 +108,16 @@ def alloc_tiled_workspace(num_chunks, rows_per_chunk, device):
 
 
 def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=None, round_mode="rtn", workspace=None,
-               grad_out=None, want_f32=False, quantize_x=False, saturate=False, kahan=None, num_head=0):
+               grad_out=None, want_f32=False, quantize_x=False, saturate=False, kahan=None, num_head=0, loss_out=None):
     """One training step of the bf16 layer (chunked.py:76-133) or of the simulated-FP8 mode of the FP8 layer
     (chunked_fp8xmc_clf.py:98-99,110,115-116), three kernels per chunk.  `chunk_views` are contiguous [rows, 768]
     tensors (views of one weight tensor, or the FP8 layer's chunk parameters): all have rows_per_chunk rows except the
     last, which may be shorter.  Updated in place; returns grad_input (bf16) or (grad_input, grad_x_fp32).
     e4m3 weights: quantize_x / saturate select the true-FP8 arithmetic (logits from e4m3(X), saturating cast) instead of
     the simulated one; `kahan` ([num_head, 768] bf16 or float8_e5m2, updated in place) turns on the head-Kahan update of
-    the first num_head rows of chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127-131)."""
+    the first num_head rows of chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127-131).  `loss_out` (a float32 device tensor
+    with one element) receives the summed binary cross entropy of the step's logits (what chunked.py:57-72 is written
+    to compute)."""
     lib = _lib.load()
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == FEATURES
     ktype = 0
@@ -143,11 +145,14 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
     sarr = None
     if seeds is not None:
         sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
+    if loss_out is not None:
+        assert loss_out.is_cuda and loss_out.dtype == torch.float32 and loss_out.numel() == 1
     st = lib.xmc_tiled_step(arr, nc, rows_per_chunk, chunk_views[-1].shape[0], WEIGHT_TYPES[weight_type], x.data_ptr(),
                             batch, FEATURES, labels.data_ptr() if labels.numel() else None, labels.shape[0], float(lr),
                             sarr, _lib.ROUND_MODES[round_mode], int(bool(quantize_x)), int(bool(saturate)),
                             kahan.data_ptr() if kahan is not None else None, ktype, int(num_head), grad_out.data_ptr(),
-                            gf.data_ptr() if gf is not None else None, workspace.data_ptr(), workspace.numel(),
+                            gf.data_ptr() if gf is not None else None,
+                            loss_out.data_ptr() if loss_out is not None else None, workspace.data_ptr(), workspace.numel(),
                             _stream_ptr())
     _lib.check(st, "xmc_tiled_step")
     return (grad_out, gf) if want_f32 else grad_out

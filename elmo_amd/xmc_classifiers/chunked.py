@@ -103,10 +103,11 @@ class XMCBCECHUNKEDLayer(nn.Module):
             embed: Encoder or bottleneck layer output, [B, 768], B <= 128 (any value).
             labels: Positive labels in sparse format (row,col). shape = (Nb,2).
             xmc_lr: list of learning rates, only [0] is used.
-            skip_loss: must be True: the reference's own non-skip branch is broken (it passes the weights where the
-                       logits belong, chunked.py:109) and the training loop never takes it.
+            skip_loss: Whether to skip the loss calculation.  When False the summed binary cross entropy of the step's
+                       logits is computed inside the logits kernel and returned (one host synchronisation).  This is
+                       the value the reference's _compute_loss is written to return (chunked.py:57-72); the reference
+                       itself passes the weight chunk where the logits belong (chunked.py:109).
         '''
-        assert skip_loss, "the loss of the chunked layer is not computed by this build (dead code in the reference)"
         assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
         assert embed.shape[0] <= ops.MAX_BATCH, "batch must be at most 128"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
@@ -120,7 +121,10 @@ class XMCBCECHUNKEDLayer(nn.Module):
         views = self._chunks()
         # one seed per chunk from the global CPU generator, as the reference draws them (chunked.py:126)
         seeds = [torch.randint(0, 1000000, (1,)).item() for _ in range(len(views))]
+        loss_out = None if skip_loss else torch.zeros(1, dtype=torch.float32, device=x.device)
         self.grad_input = ops.tiled_step(views, self.chunk_size, "bf16", x, lab, xmc_lr[0], seeds=seeds,
-                                         round_mode=self.rounding, workspace=self._workspace)
+                                         round_mode=self.rounding, workspace=self._workspace, loss_out=loss_out)
         self.iteration += 1
+        if loss_out is not None:
+            loss = loss_out.item()
         return loss

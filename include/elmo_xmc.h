@@ -105,12 +105,17 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk);
  *                    head-Kahan update of Fp8XMCBCEChunkedHeadKahanLayer (chunked_head_kahan_fp8xmc_clf.py:41-48,127-131;
  *                    fuse_kernel.py:202-262), e4m3 weights only: device buffer [num_head, 768] of bf16 (kahan_type 1) or
  *                    e5m2 (kahan_type 2) for the first num_head rows of chunk 0, updated in place; kahan_type 0 = none
+ *   loss_out         device float or null.  Not null: receives the summed binary cross entropy of the step's bf16 logits
+ *                    against the targets, sum over labels and batch rows of max(z,0) - [positive] z + log(1 + exp(-|z|)),
+ *                    which is what _compute_loss of the reference is written to return (chunked.py:57-72; its caller
+ *                    passes the weights where the logits belong, chunked.py:109, so the reference itself never returns
+ *                    this value).  fp32 per element, summed in a fixed order.
  */
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
                    const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
                    const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
-                   int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes,
-                   void* stream);
+                   int num_head, void* grad_x_bf16, float* grad_x_f32, float* loss_out, void* workspace,
+                   size_t workspace_bytes, void* stream);
 
 /* Selects the fused kernel that xmc_fp8_step launches (no counterpart in the reference): 0 = four compute units per
  * tile stream without repeated arithmetic (default), 1 = two compute units per tile stream with the logits computed

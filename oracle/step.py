@@ -179,14 +179,15 @@ def fp8_forward(w_codes, x_any, num_labels, *, simulated=False, scale_w=1.0, sca
     return np.concatenate(outs, axis=1)[:, :num_labels]
 
 
-def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rtn", return_parts=False):
+def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rtn", return_parts=False,
+              return_loss=False):
     """One step of the bf16 layer (chunked.py:85-131), weights bf16.
 
     w_bf16 : fp32 array [L, d] holding bf16 values (single tensor, chunk views of ceil(L/nc) rows, last short)
     sr_mode: "rtn"        W' = bf16(f32(W) - lr*f32(A))
              "reference"  W' = SR16(f32(W) - f32(A)*lr; philox(seed_c, flat idx in chunk))  (stochastic_rounding_kernel.py:80-89)
     Weight decay is ignored exactly as the bf16 path of the reference ignores it (:91-99).
-    Returns (new_w [L,d] bf16-valued fp32, gx_fp32 [B,d], grad_input bf16-valued fp32).
+    Returns (new_w [L,d] bf16-valued fp32, gx_fp32 [B,d], grad_input bf16-valued fp32[, loss with return_loss]).
     """
     w_all = np.ascontiguousarray(w_bf16, dtype=np.float32)
     x = np.ascontiguousarray(x_bf16, dtype=np.float32)
@@ -198,6 +199,7 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
     gx = np.zeros((B, d), dtype=np.float32)
     new_w = w_all.copy()
     parts = []
+    loss = 0.0
     for c in range(num_chunks):
         lo, hi = c * cs, min((c + 1) * cs, L)
         if lo >= hi:
@@ -207,6 +209,7 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
         z = (x64 @ w64.T).astype(np.float32)                        # [B, L_c]  (:101)
         pos = _positives_mask(labels, B, lo, hi).T
         zb, g = _grad_from_logits(z, pos)                           # (:112-113)
+        loss += bce_loss_sum(zb, pos)
         g64 = g.astype(np.float64)
         gx = gx + C.bf16_round((g64 @ w64).astype(np.float32))      # partial rounded to bf16 (:116)
         a = C.bf16_round((g64.T @ x64).astype(np.float32))          # materialised bf16 grad (:119)
@@ -223,7 +226,16 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
         if return_parts:
             parts.append(dict(z=zb, g=g, a=a, t=t))
     out = (new_w, gx, C.bf16_round(gx))
+    if return_loss:
+        out = out + (loss,)
     return out + (parts,) if return_parts else out
+
+
+def bce_loss_sum(z_bf16, posmask):
+    """Summed binary cross entropy with logits, the quantity chunked.py:57-72 is written to return when it is handed
+    the logits: sum(max(z,0)) - sum(z at positives) + sum(log(1 + exp(-|z|))).  float64; z are the bf16 logits."""
+    z = np.asarray(z_bf16, dtype=np.float64)
+    return float(np.maximum(z, 0.0).sum() - z[np.asarray(posmask, dtype=bool)].sum() + np.log1p(np.exp(-np.abs(z))).sum())
 
 
 def bf16_forward(w_bf16, x_bf16):

@@ -174,3 +174,36 @@ def test_kahan_step_invariants():
     c8, k8, _, _ = O.fp8_kahan_step(case["chunks"], kz, x, labels, 0.05, nh, kahan_type="e5m2", sr_mode="rtn")
     cb, kb, _, _ = O.fp8_kahan_step(case["chunks"], np.zeros((nh, 768), np.float32), x, labels, 0.05, nh, sr_mode="rtn")
     assert np.array_equal(c8[0], cb[0]) and np.abs(C.e5m2_decode(k8) - kb).max() <= 2.0 ** -3 * np.abs(kb).max()
+
+
+def test_loss_matches_the_library_routine_and_the_cited_op_sequence():
+    """bce_loss_sum against torch's binary_cross_entropy_with_logits (float64, sum) and against the operations of
+    chunked.py:61-72 restated one by one in fp32; and the step's loss against the same routine on the oracle's logits."""
+    import torch
+    rng = np.random.default_rng(5)
+    z = C.bf16_round(rng.normal(0, 3.0, size=(40, 24)).astype(np.float32))
+    pos = rng.random((40, 24)) < 0.1
+    want = torch.nn.functional.binary_cross_entropy_with_logits(
+        torch.from_numpy(z.astype(np.float64)), torch.from_numpy(pos.astype(np.float64)), reduction="sum").item()
+    got = O.bce_loss_sum(z, pos)
+    assert abs(got - want) <= 1e-9 * abs(want)
+    zt = torch.from_numpy(z)
+    rows, cols = np.nonzero(pos)
+    temp = zt.clone().clamp_(min=0.0)
+    seq = temp.sum() - zt[rows, cols].sum()
+    temp = zt.clone().abs_().neg_().exp_().add_(1.0).log_()
+    seq = (seq + temp.sum()).item()
+    assert abs(got - seq) <= 1e-5 * abs(want)
+    assert O.bce_loss_sum(np.zeros((3, 2)), np.zeros((3, 2), bool)) == pytest.approx(6 * np.log(2.0))
+
+    # the step: 70 labels in 2 chunks, batch 8
+    x = synth.make_x(8, 768, 9)
+    w = C.bf16_round(synth.make_weights_np(70, 768, 9, 0.5))
+    labels = synth.make_labels(8, 70, 3.0, 1.0, 9)
+    _, _, _, loss, parts = O.bf16_step(w, x, labels, 0.05, 2, sr_mode="rtn", return_loss=True, return_parts=True)
+    zall = np.concatenate([p["z"] for p in parts], axis=1)          # [B, L]
+    y = np.zeros_like(zall)
+    y[labels[:, 0], labels[:, 1]] = 1.0
+    want = torch.nn.functional.binary_cross_entropy_with_logits(
+        torch.from_numpy(zall.astype(np.float64)), torch.from_numpy(y.astype(np.float64)), reduction="sum").item()
+    assert abs(loss - want) <= 1e-9 * abs(want)

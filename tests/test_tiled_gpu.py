@@ -85,6 +85,30 @@ def test_bf16_layer_reference_stochastic_rounding(gpu):
     assert (new2 != new).mean() > 0.1
 
 
+def test_loss_of_a_ragged_case_with_large_logits(gpu):
+    """Loss fused into the logits kernel: ragged chunks, batch not a multiple of 16, weights large enough that the
+    logits leave the linear range of the softplus; padded batch rows and rows past the chunk must not count."""
+    import torch
+    from elmo_amd import ops
+    L, nc, batch = 1000, 3, 24
+    w = C.bf16_round(synth.make_weights_np(L, 768, 41, 2.0))
+    x = synth.make_x(batch, 768, 41)
+    labels = synth.make_labels(batch, L, 6.0, 1.0, 41)
+    wt = torch.from_numpy(C.bf16_bits(w).view(np.int16)).to(gpu).view(torch.bfloat16)
+    xt = torch.from_numpy(C.bf16_bits(x).view(np.int16)).to(gpu).view(torch.bfloat16)
+    lt = torch.from_numpy(labels).to(gpu)
+    cs = (L + nc - 1) // nc
+    views = [wt[c * cs:min((c + 1) * cs, L)] for c in range(nc)]
+    loss = torch.zeros(1, dtype=torch.float32, device=gpu)
+    ops.tiled_step(views, cs, "bf16", xt, lt, 0.0, round_mode="rtn", loss_out=loss)
+    _, _, _, ref_loss = O.bf16_step(w, x, labels, 0.0, nc, sr_mode="rtn", return_loss=True)
+    assert abs(loss.item() - ref_loss) <= 1e-4 * abs(ref_loss), (loss.item(), ref_loss)
+    # a second call gives the same bits (fixed summation order)
+    loss2 = torch.zeros(1, dtype=torch.float32, device=gpu)
+    ops.tiled_step(views, cs, "bf16", xt, lt, 0.0, round_mode="rtn", loss_out=loss2)
+    assert loss.item() == loss2.item()
+
+
 def test_bf16_layer_duplicates_and_no_positives(gpu):
     x, w, labels = bf16_case(640, 16, 51)
     dup = np.array([[0, 5], [0, 5], [3, 639], [3, 639], [15, 0]], dtype=np.int32)
@@ -177,6 +201,13 @@ def test_chunked_module_contract(gpu):
     assert enc.weight.grad is not None
     logits = xfc.xfc_forward(tokens)
     assert logits.shape == (24, 1000)
+    # skip_loss=False: the summed binary cross entropy of the step's logits (what chunked.py:57-72 is written to return)
+    w1 = xfc.xfc_weight.float().cpu().numpy()
+    out2 = enc(tokens)
+    loss = xfc.xfc_forward_backward(out2, labels, [0.05], skip_loss=False)
+    _, _, _, ref_loss = O.bf16_step(w1, out2.detach().float().cpu().numpy(), labels.cpu().numpy(), 0.05, 3, sr_mode="rtn",
+                                    return_loss=True)
+    assert isinstance(loss, float) and abs(loss - ref_loss) <= 1e-4 * abs(ref_loss), (loss, ref_loss)
     with pytest.raises(AssertionError):
         cfg2 = make_cfg("cuda:0", 1000, 3)
         cfg2.model.xmc.dtype = "float32"
