@@ -231,12 +231,13 @@ int xmc_profile_events(void* start_event, void* stop_event) {
   return XMC_OK;
 }
 
-size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk) {
-  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
+size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_batch) {
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0 || max_batch <= 0 || max_batch > T_HALVES * BP) return 0;
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
-  // G in both orientations, tile_ptr (padded to 64 entries), one loss share per tile
-  return TW_G + 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 4 + 255) / 256 * 256;
+  const size_t halves = ((size_t)max_batch + BP - 1) / BP;
+  // per batch half G in both orientations; tile_ptr (padded to 64 entries); one loss share per tile
+  return TW_G + halves * 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 4 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
@@ -248,7 +249,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (kahan_type < 0 || kahan_type > 2 || (kahan_type != 0 && (weight_type != W_E4M3 || !kahan))) return XMC_ERR_MODE;
   if (kahan_type != 0 && (num_head < 0 || num_head > rows_per_chunk || !aligned16(kahan))) return XMC_ERR_SHAPE;
   if (kahan_type == 0) num_head = 0;
-  if (features != D || batch <= 0 || batch > BP) return XMC_ERR_SHAPE;
+  if (features != D || batch <= 0 || batch > T_HALVES * BP) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_last_chunk <= 0 || rows_last_chunk > rows_per_chunk) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
   if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1 || nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
@@ -260,7 +261,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
   }
   if (!aligned16(x_bf16) || ((uintptr_t)workspace & 255) != 0) return XMC_ERR_ALIGN;
-  if (workspace_bytes < xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk)) return XMC_ERR_WORKSPACE;
+  if (workspace_bytes < xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk, batch)) return XMC_ERR_WORKSPACE;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;
   hipStream_t stream = (hipStream_t)stream_;
@@ -274,9 +275,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   unsigned* keys = (unsigned*)(ws + TW_KEYS);
   float* gx_total = (float*)(ws + TW_GX);
   floatx4* partial = (floatx4*)(ws + TW_PART);
+  const int halves = (batch + BP - 1) / BP;
+  const size_t g_half = 2 * (size_t)rows_pad * BP;    // elements of one half's G and G^T
   unsigned short* glb = (unsigned short*)(ws + TW_G);
   unsigned short* gbl = glb + (size_t)rows_pad * BP;
-  int* tile_ptr = (int*)(gbl + (size_t)rows_pad * BP);
+  int* tile_ptr = (int*)(glb + halves * g_half);
   float* loss_part = (float*)(tile_ptr + (num_tiles + 1 + 63) / 64 * 64);   // one share per tile
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
@@ -284,8 +287,8 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (n_pad > 0)
     quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys, nullptr);
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
-  tiled_prep_x_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, quantize_x, xb, xT);
-  tiled_zero_kernel<<<(BP * D + 255) / 256, 256, 0, stream>>>(gx_total, BP * D);
+  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT);
+  tiled_zero_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>(gx_total, halves * BP * D);
   if (loss_out) tiled_zero_kernel<<<(num_tiles + 255) / 256, 256, 0, stream>>>(loss_part, num_tiles);
   for (int c = 0; c < num_chunks; c++) {
     void* w = chunk_ptrs[c];
@@ -300,22 +303,28 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int splits = (rp + range - 1) / range;
     const int* tp = tile_ptr + c * tiles_per_chunk;
     float* lp = loss_part + c * tiles_per_chunk;
-    if (weight_type == W_BF16) {
-      if (loss_out) tiled_logits_kernel<W_BF16, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
-      else tiled_logits_kernel<W_BF16, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
-      tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
-    } else {
-      if (loss_out) tiled_logits_kernel<W_E4M3, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
-      else tiled_logits_kernel<W_E4M3, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xb, keys, tp, label0, glb, gbl, batch, lp);
-      tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gbl, partial);
+    for (int hh = 0; hh < halves; hh++) {
+      unsigned short* gl = glb + hh * g_half;
+      unsigned short* gb = gbl + hh * g_half;
+      const unsigned short* xh = xb + (size_t)hh * BP * D;
+      const unsigned brow0 = (unsigned)(hh * BP);
+      if (weight_type == W_BF16) {
+        if (loss_out) tiled_logits_kernel<W_BF16, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        else tiled_logits_kernel<W_BF16, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
+      } else {
+        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        else tiled_logits_kernel<W_E4M3, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
+      }
+      tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
-    tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total);
     if (weight_type == W_BF16) {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
-      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
     } else {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
-      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
     }
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);

@@ -18,13 +18,16 @@ constexpr int T_WS2 = 48 * 2 + 16;                 // LDS row stride of a wavefr
 typedef short tshortx4 __attribute__((ext_vector_type(4)));
 typedef short tshortx8 __attribute__((ext_vector_type(8)));
 
+// The batch is processed in halves of up to 128 rows (T_HALVES of them at most): logits and grad_X per half, grad_W summed
+// over the halves.
+constexpr int T_HALVES = 2;
 // workspace of the tiled path (byte offsets, 256-byte aligned)
-constexpr size_t TW_XB = 0;                                        // X   [128][768] bf16, rows beyond the batch zero
-constexpr size_t TW_XT = TW_XB + (size_t)BP * D * 2;               // X^T [768][128] bf16
-constexpr size_t TW_KEYS = TW_XT + (size_t)BP * D * 2;             // sorted positive keys
-constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [128][768]
-constexpr size_t TW_PART = TW_GX + (size_t)BP * D * 4;             // grad_X partials [T_SPLITS][128*768] fp32
-constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // G [rows_pad][128] then G^T [128][rows_pad], then tile_ptr
+constexpr size_t TW_XB = 0;                                        // X   [halves][128][768] bf16, rows beyond the batch zero
+constexpr size_t TW_XT = TW_XB + (size_t)T_HALVES * BP * D * 2;    // X^T [halves][768][128] bf16
+constexpr size_t TW_KEYS = TW_XT + (size_t)T_HALVES * BP * D * 2;  // sorted positive keys
+constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [halves*128][768]
+constexpr size_t TW_PART = TW_GX + (size_t)T_HALVES * BP * D * 4;  // grad_X partials [T_SPLITS][128*768] fp32 (one half at a time)
+constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // per half: G [rows_pad][128] then G^T [128][rows_pad]; then tile_ptr
 
 __device__ __forceinline__ bf16x8 t_fp8x8_to_bf16x8(intx2 raw) {
   bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
@@ -41,9 +44,9 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 
 // X -> zero-padded row-major image (for the logits; optionally quantised to e4m3 and widened back, which makes the bf16
 // products equal to the FP8 ones of chunked_fp8xmc_clf.py:101-102) and its transpose (for grad_W, never quantised)
-__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int quantize, unsigned short* xb, unsigned short* xT) {
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= BP * D) return;
+  if (i >= halves * BP * D) return;
   int b = i / D, k = i - b * D;
   unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
   unsigned short vq = v;
@@ -54,7 +57,7 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int quan
     vq = bf16_bits(back.x);
   }
   xb[i] = vq;
-  xT[(size_t)k * BP + b] = v;
+  xT[((size_t)(b >> 7) * D + k) * BP + (b & 127)] = v;
 }
 
 __global__ void tiled_zero_kernel(float* p, int n) {
@@ -71,7 +74,8 @@ __global__ void tiled_zero_kernel(float* p, int n) {
 template <int WT, bool LOSS>
 __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int rows, int rows_pad, const unsigned short* xb,
                                                            const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
-                                                           unsigned short* glb, unsigned short* gbl, int batch, float* loss_part) {
+                                                           unsigned short* glb, unsigned short* gbl, int batch, unsigned brow0,
+                                                           float* loss_part) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int r0 = blockIdx.x * TL + 16 * wv;
   const int lrow = min(r0 + l16, rows - 1);
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
       sg[nb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + ex));
       if (LOSS) {
         acc[nb][e] = zf;   // kept for the positives below
-        if (r0 + 4 * kg + e < rows && 16 * nb + l16 < batch)
+        if (r0 + 4 * kg + e < rows && (int)brow0 + 16 * nb + l16 < batch)
           lsum += __builtin_fmaxf(zf, 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf) * 1.44269504088896340736f));
       }
     }
@@ -111,8 +115,8 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
     const unsigned key = keys[e];
     const unsigned prev = e > 0 ? keys[e - 1] : ~key;
     const unsigned l = (key >> 8) - lbase;
-    const unsigned b = key & 255u;
-    if (prev != key && l < 4u && (b & 15u) == (unsigned)l16) {
+    const unsigned b = (key & 255u) - brow0;   // batch row within this half
+    if (prev != key && l < 4u && b < (unsigned)BP && (b & 15u) == (unsigned)l16) {
 #pragma unroll
       for (int nb = 0; nb < 8; nb++)
 #pragma unroll
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
     for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
     if (lane == 0) wsum[wv] = lsum;
     __syncthreads();
-    if (tid == 0) loss_part[blockIdx.x] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+    if (tid == 0) loss_part[blockIdx.x] += (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);   // the halves run one after the other
   }
 #pragma unroll
   for (int nb = 0; nb < 8; nb++) {
@@ -261,23 +265,31 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 //                       k' = ((k + w) - W') - lr*A stored as bf16 (kahan_type 1) or e5m2 (2); rows behind the head take
 //                       their random offsets from (row - num_head), as the reference's call on the sliced tensors does
 template <int WT, int MODE>
-__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, const unsigned short* xT,
-                                                           float lr, unsigned seed, int saturate, void* kahan, int kahan_type,
-                                                           int num_head) {
+__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, size_t g_half_stride,
+                                                           int halves, const unsigned short* xT, float lr, unsigned seed,
+                                                           int saturate, void* kahan, int kahan_type, int num_head) {
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, tile = blockIdx.x >> 2;
   const int row = tile * TL + 16 * wv + l16;
-  bf16x8 gf[4];
+  bf16x8 gf[T_HALVES][4];
 #pragma unroll
-  for (int ks = 0; ks < 4; ks++) gf[ks] = *(const bf16x8*)(glb + (size_t)row * BP + 32 * ks + 8 * kg);
+  for (int hh = 0; hh < T_HALVES; hh++)
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
+      gf[hh][ks] = hh < halves ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
 #pragma unroll 2
   for (int nn = 0; nn < 12; nn++) {
     const int f = 192 * fb + 16 * nn;
     floatx4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      const bf16x8 xa = *(const bf16x8*)(xT + (size_t)(f + l16) * BP + 32 * ks + 8 * kg);
-      a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[ks], a, 0, 0, 0);
+    for (int hh = 0; hh < T_HALVES; hh++) {
+      if (hh < halves) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+          const bf16x8 xa = *(const bf16x8*)(xT + ((size_t)hh * D + f + l16) * BP + 32 * ks + 8 * kg);
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
+        }
+      }
     }
     // a[e] = A[label row][feature f + 4kg + e]
     if (row < rows) {

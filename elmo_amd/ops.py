@@ -6,7 +6,8 @@ import torch
 from . import _lib
 
 FEATURES = 768
-MAX_BATCH = 128
+MAX_BATCH = 128          # fused step
+MAX_BATCH_TILED = 256    # three-kernel step
 
 
 def _stream_ptr():
@@ -96,15 +97,15 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
 WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}
 
 
-def tiled_workspace_bytes(num_chunks, rows_per_chunk):
-    n = _lib.load().xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk)
+def tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch=MAX_BATCH):
+    n = _lib.load().xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch)
     if n == 0:
         raise _lib.XmcError("unsupported chunk geometry")
     return n
 
 
-def alloc_tiled_workspace(num_chunks, rows_per_chunk, device):
-    return torch.empty(tiled_workspace_bytes(num_chunks, rows_per_chunk), dtype=torch.uint8, device=device)
+def alloc_tiled_workspace(num_chunks, rows_per_chunk, device, max_batch=MAX_BATCH):
+    return torch.empty(tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch), dtype=torch.uint8, device=device)
 
 
 def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=None, round_mode="rtn", workspace=None,
@@ -136,9 +137,9 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
         assert c.shape[0] == rows_per_chunk or (i == nc - 1 and 0 < c.shape[0] <= rows_per_chunk)
         arr[i] = c.data_ptr()
     batch = x.shape[0]
-    assert 0 < batch <= MAX_BATCH, "batch must be at most 128"
-    if workspace is None:
-        workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device)
+    assert 0 < batch <= MAX_BATCH_TILED, "batch must be at most 256"
+    if workspace is None or workspace.numel() < tiled_workspace_bytes(nc, rows_per_chunk, batch):
+        workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device, batch)
     if grad_out is None:
         grad_out = torch.empty(batch, FEATURES, dtype=torch.bfloat16, device=x.device)
     gf = torch.empty(batch, FEATURES, dtype=torch.float32, device=x.device) if want_f32 else None

@@ -67,7 +67,8 @@ class XMCBCECHUNKEDLayer(nn.Module):
         self.dummy = torch.zeros(1, dtype=self._dtype, device=self.device)
         self.loss = torch.tensor(0.0, device=self.device)
         self.iteration = 0
-        self._workspace = ops.alloc_tiled_workspace(self.num_chunks, self.chunk_size, self.device)
+        self._workspace = ops.alloc_tiled_workspace(self.num_chunks, self.chunk_size, self.device,
+                                                    min(max(int(cfg.data.batch_size), ops.MAX_BATCH), ops.MAX_BATCH_TILED))
 
     def _chunks(self):
         w = self.xfc_weight
@@ -100,7 +101,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
         '''
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args:
-            embed: Encoder or bottleneck layer output, [B, 768], B <= 128 (any value).
+            embed: Encoder or bottleneck layer output, [B, 768], B <= 256 (any value).
             labels: Positive labels in sparse format (row,col). shape = (Nb,2).
             xmc_lr: list of learning rates, only [0] is used.
             skip_loss: Whether to skip the loss calculation.  When False the summed binary cross entropy of the step's
@@ -109,7 +110,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
                        itself passes the weight chunk where the logits belong (chunked.py:109).
         '''
         assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
-        assert embed.shape[0] <= ops.MAX_BATCH, "batch must be at most 128"
+        assert embed.shape[0] <= ops.MAX_BATCH_TILED, "batch must be at most 256"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
         x = embed.detach()
         if x.dtype != self._dtype:

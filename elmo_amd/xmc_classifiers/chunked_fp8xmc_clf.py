@@ -80,9 +80,13 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         # all scratch memory of the step comes from the torch allocator (so that max_memory_allocated sees it)
         self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
         self._tiled_workspace = None
+        # batches of more than 128 rows (up to 256) also run on the three-kernel path, with the true-FP8 arithmetic
+        self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "simulated FP8 has no per-tensor scales"
-            self._tiled_workspace = ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device)
+        if self.fake_fp8_matmul or self._max_batch > ops.MAX_BATCH:
+            self._tiled_workspace = ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device,
+                                                              min(max(self._max_batch, ops.MAX_BATCH), ops.MAX_BATCH_TILED))
 
     def _chunks(self):
         return [w.data for w in self.xfc_weight]
@@ -111,14 +115,15 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         '''
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args:
-            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 128.
+            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 256 (the fused
+                   kernel takes up to 128 rows, larger batches run on the three-kernel path).
             labels: Positive labels in sparse format, int32 [Nb, 2] = (row in batch, label id).
             xmc_lr: list of learning rates, only [0] is used.
             skip_loss: ignored, as in the reference's FP8 layer; the return value is 0.
         '''
         assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
-        assert embed.shape[0] <= ops.MAX_BATCH and (self.fake_fp8_matmul or embed.shape[0] % 16 == 0), \
-            "batch must be a multiple of 16 and at most 128 (the reference data loader uses drop_last)"
+        assert embed.shape[0] <= ops.MAX_BATCH_TILED and (self.fake_fp8_matmul or embed.shape[0] % 16 == 0), \
+            "batch must be a multiple of 16 and at most 256 (the reference data loader uses drop_last)"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
         x = embed.detach()
         if x.dtype != torch.bfloat16:
@@ -132,6 +137,14 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace)
+        elif embed.shape[0] > ops.MAX_BATCH:
+            # the fused kernel holds 128 batch rows; larger batches take the three-kernel path with the same arithmetic
+            # (logits from e4m3(X), saturating cast), which rounds with the reference's recipe or to nearest
+            assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128"
+            mode = "rtn" if self.rounding == "rtn" else "sr_philox"
+            self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
+                                             round_mode=mode, workspace=self._tiled_workspace, quantize_x=True,
+                                             saturate=True)
         else:
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
                                            scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)

@@ -85,8 +85,8 @@ enum {
   XMC_WEIGHT_BF16 = 1       /* bf16 layer (chunked.py:85-131) */
 };
 
-/* Bytes of workspace xmc_tiled_step needs. */
-size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk);
+/* Bytes of workspace xmc_tiled_step needs for batches of up to max_batch rows (1..256). */
+size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_batch);
 
 /* One training step of the modes in which the reference keeps bf16 temporaries, three kernels per chunk as there:
  *   XMC_WEIGHT_BF16  XMCBCECHUNKEDLayer.xfc_forward_backward (chunked.py:76-133) with sgd_update
@@ -98,7 +98,7 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk);
  *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
- *   round_mode       XMC_ROUND_RTN or XMC_ROUND_SR_PHILOX; batch: 1..128, any value
+ *   round_mode       XMC_ROUND_RTN or XMC_ROUND_SR_PHILOX; batch: 1..256, any value (processed in halves of 128 rows)
  *   quantize_x       e4m3 weights: 0 = logits from the un-quantised X (simulated FP8), 1 = from e4m3(X) (true FP8, :101)
  *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
  *   kahan, kahan_type, num_head

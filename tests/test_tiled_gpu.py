@@ -59,6 +59,8 @@ def check_gx(gf, gb, ref_gx, tol=1e-3):
     (1000, 3, 24, 32),          # ragged chunks (334, 334, 332), batch not a multiple of 16
     (5000, 2, 128, 33),         # full batch
     (20011, 4, 64, 34),         # prime label count
+    (3000, 2, 200, 35),         # two batch halves, the second one short
+    (1500, 3, 256, 36),         # the largest batch
 ])
 def test_bf16_layer_rtn_parity(gpu, L, nc, batch, seed):
     x, w, labels = bf16_case(L, batch, seed)
@@ -291,6 +293,42 @@ def test_true_fp8_on_the_tiled_path_matches_the_fused_oracle(gpu):
         d = H.e4m3_ulp_distance(a, b)
         assert d.max() <= 1 and (d != 0).mean() < 2e-3
     check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx)
+
+
+def test_true_fp8_with_a_batch_of_256(gpu):
+    """Batches above 128 rows run on the three-kernel path in two halves: logits and grad_X per half, grad_W over both."""
+    import torch
+    from elmo_amd import ops
+    case = H.make_case(2, 1024, 256, 61, pos_mean=4.0, extra_labels=[[255, 2047], [128, 0], [127, 0], [200, 1000], [200, 1000]])
+    chunks, x, labels = H.to_device_case(case, gpu)
+    g, gf = ops.tiled_step(chunks, 1024, "e4m3", x, labels, 0.05, round_mode="rtn", want_f32=True, quantize_x=True, saturate=True)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn")
+    new = H.chunks_to_numpy(chunks)
+    mism = total = 0
+    for a, b in zip(new, ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1
+        mism += int((d != 0).sum()); total += d.size
+    assert mism / total < 2e-3
+    assert gf.shape == (256, 768)
+    assert np.abs(gf.cpu().numpy() - ref_gx).max() <= 1e-3 * np.abs(ref_gx).max()
+
+    # the module routes such a batch there by itself
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked_fp8xmc_clf import Fp8XMCBCEChunkedLayer
+    cfg = make_cfg("cuda:0", 2000, 2, rounding="rtn")
+    cfg.data.batch_size = 256
+    torch.manual_seed(3)
+    xfc = Fp8XMCBCEChunkedLayer(cfg)
+    w0 = [w.data.view(torch.uint8).cpu().numpy() for w in xfc.xfc_weight]
+    emb = torch.from_numpy(C.bf16_bits(synth.make_x(256, 768, 62)).view(np.int16)).to(gpu).view(torch.bfloat16)
+    lab = torch.from_numpy(synth.make_labels(256, 2000, 4.0, 1.0, 62)).to(gpu)
+    assert xfc.xfc_forward_backward(emb, lab, [0.05]) == 0
+    ref_codes, ref_gx, ref_gi = O.fp8_step(w0, emb.float().cpu().numpy(), lab.cpu().numpy(), 0.05, sr_mode="rtn")
+    for wt, b in zip(xfc.xfc_weight, ref_codes):
+        assert H.e4m3_ulp_distance(wt.data.view(torch.uint8).cpu().numpy(), b).max() <= 1
+    assert xfc.grad_input.shape == (256, 768)
+    H.assert_bf16_close(xfc.grad_input.float().cpu().numpy(), ref_gi)
 
 
 def test_head_kahan_module(gpu):
