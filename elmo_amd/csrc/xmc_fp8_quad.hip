@@ -69,11 +69,11 @@ struct QuadParams {
   int rows_per_chunk;
   int tiles_per_chunk;
   int num_tiles;
-  const unsigned char* xq;            // logits operands (prep_x_quad_kernel layout)
+  const unsigned char* xq;            // logits operands (layout of prep_x_quad_thread)
   const bf16x8* xt;                   // grad_W operands
   const unsigned* keys;               // sorted positives: label*256 + batch_row
   const int* tile_ptr;                // [num_tiles+1] offsets into keys
-  const uint4* desc;                  // [num_tiles][2] tile descriptors written by tile_desc_kernel
+  const uint4* desc;                  // [num_tiles][2] tile descriptors written by quad_desc_prep_kernel
   floatx4* partial;                   // [gridDim.x][12][512] per-workgroup grad_X partial sums
   unsigned char* exch;                // [nquads][QSLOTS][QG_BYTES] G exchange ring
   int* flags;                         // [nquads][4] tiles-published counters; [nquads*4] error word; then xcc ids
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     q_lds_load16_l2(gsrc_lane + (i & (QSLOTS - 1)) * QG_BYTES + s * 8192, (unsigned)(QLDS_G + slot * QG_BYTES + (v + 8 * s) * 1024));
   };
   // snapshot of the four counters of iteration i (wavefront 0 only), read in the next iteration
-  auto issue_mailbox = [&](int i) {
+  auto issue_snapshot = [&](int i) {
     if (v != 0) return;
     if (lane < 4) q_lds_load4_l2(flags + lane, (unsigned)(QLDS_M + (i & 1) * 16));
   };
@@ -461,7 +461,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     // G of the positions up to i+QAHEAD-2 was stored in iteration i-2 or earlier: complete by the wait above
     if (tid == 0 && i >= 2 && i + QAHEAD - 1 <= n_it)
       __hip_atomic_store(flags + m, i + QAHEAD - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    issue_mailbox(i);
+    issue_snapshot(i);
     if (i + 1 < n_it) wait_published(i + 2, fmin);
     // the loads of this iteration, one at a time between the phases below
     auto mem_piece = [&](int k) {
