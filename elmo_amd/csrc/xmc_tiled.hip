@@ -42,8 +42,12 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
   return t_fp8x8_to_bf16x8(*(const intx2*)((const unsigned char*)w + idx));
 }
 
-// X -> zero-padded row-major image (for the logits; optionally quantised to e4m3 and widened back, which makes the bf16
-// products equal to the FP8 ones of chunked_fp8xmc_clf.py:101-102) and its transpose (for grad_W, never quantised)
+// X -> two zero-padded images per batch half, both in the order in which v_mfma_f32_16x16x32_bf16 takes its operands
+// (element j of lane l16 + 16 kg is row l16, k = 8 kg + j of a 16 x 32 block), so that a wavefront's operand load is
+// 1 KiB of consecutive bytes:
+//   xb: X for the logits (optionally quantised to e4m3 and widened back, which makes the bf16 products equal to the FP8
+//       ones of chunked_fp8xmc_clf.py:101-102): block (nb, ks) = batch rows 16nb.. x features 32ks..
+//   xT: X^T for grad_W (never quantised): block (fblk, ks) = features 16fblk.. x batch rows 32ks..
 __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
@@ -56,8 +60,9 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
     const floatx2 back = __builtin_amdgcn_cvt_pk_f32_fp8(code, false);
     vq = bf16_bits(back.x);
   }
-  xb[i] = vq;
-  xT[((size_t)(b >> 7) * D + k) * BP + (b & 127)] = v;
+  const int half = b >> 7, bh = b & 127;
+  xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
+  xT[(size_t)half * BP * D + ((size_t)((k >> 4) * (BP / 32) + (bh >> 5)) * 64 + (k & 15) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
 }
 
 __global__ void tiled_zero_kernel(float* p, int n) {
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
     const bf16x8 a = t_load_w8<WT>(w, (size_t)lrow * D + 32 * ks + 8 * kg);
 #pragma unroll
     for (int nb = 0; nb < 8; nb++) {
-      const bf16x8 b = *(const bf16x8*)(xb + (size_t)(16 * nb + l16) * D + 32 * ks + 8 * kg);
+      const bf16x8 b = *(const bf16x8*)(xb + ((size_t)(nb * (D / 32) + ks) * 64 + lane) * 8);
       acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nb], 0, 0, 0);
     }
   }
@@ -145,7 +150,8 @@ __global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int ro
     uint2 o;
     o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
     o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
-    *(uint2*)(gbl + (size_t)b * rows_pad + r0 + 4 * kg) = o;
+    // G^T in operand order for grad_X: block (label / 32, nb) of 16 batch rows x 32 labels
+    *(uint2*)(gbl + ((size_t)((blockIdx.x * 2 + (wv >> 1)) * 8 + nb) * 64 + l16 + 16 * (2 * (wv & 1) + (kg >> 1))) * 8 + 4 * (kg & 1)) = o;
 #pragma unroll
     for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
   }
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
     }
     bf16x8 ga[8];
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gbl + (size_t)(16 * mb + l16) * rows_pad + l0 + 8 * kg);
+    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gbl + ((size_t)((l0 >> 5) * 8 + mb) * 64 + lane) * 8);
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
@@ -286,7 +292,7 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
       if (hh < halves) {
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-          const bf16x8 xa = *(const bf16x8*)(xT + ((size_t)hh * D + f + l16) * BP + 32 * ks + 8 * kg);
+          const bf16x8 xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((f >> 4) * (BP / 32) + ks) * 64 + lane) * 8);
           a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
         }
       }
