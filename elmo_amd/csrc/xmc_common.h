@@ -63,8 +63,10 @@ __device__ __forceinline__ unsigned philox_word0(unsigned off, unsigned k0, unsi
   unsigned c0 = off, c1 = 0, c2 = 0, c3 = 0;
 #pragma unroll
   for (int r = 0; r < 10; r++) {
-    unsigned hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-    unsigned hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    // one 32 x 32 -> 64 bit multiply per product (both halves are needed)
+    const unsigned long long p0 = (unsigned long long)0xD2511F53u * (unsigned long long)c0;
+    const unsigned long long p1 = (unsigned long long)0xCD9E8D57u * (unsigned long long)c2;
+    const unsigned hi0 = (unsigned)(p0 >> 32), lo0 = (unsigned)p0, hi1 = (unsigned)(p1 >> 32), lo1 = (unsigned)p1;
     c0 = hi1 ^ c1 ^ k0; c1 = lo1; c2 = hi0 ^ c3 ^ k1; c3 = lo0;
     k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
   }

@@ -47,7 +47,8 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 // 1 KiB of consecutive bytes:
 //   xb: X for the logits (optionally quantised to e4m3 and widened back, which makes the bf16 products equal to the FP8
 //       ones of chunked_fp8xmc_clf.py:101-102): block (nb, ks) = batch rows 16nb.. x features 32ks..
-//   xT: X^T for grad_W (never quantised): block (fblk, ks) = features 16fblk.. x batch rows 32ks..
+//   xT: X^T for grad_W (never quantised): block (fblk, ks) = 16 features x batch rows 32ks.., the features of a block
+//       chosen so that a lane of the update kernel owns consecutive ones
 __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
@@ -62,7 +63,9 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
   }
   const int half = b >> 7, bh = b & 127;
   xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
-  xT[(size_t)half * BP * D + ((size_t)((k >> 4) * (BP / 32) + (bh >> 5)) * 64 + (k & 15) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
+  // feature k = 192 fbk + 48 kgk + 4 nn + e sits in row 4 kgk + e of block 12 fbk + nn (see tiled_update_kernel)
+  const int fbk = k / 192, r = k - fbk * 192, kgk = r / 48, nn = (r - kgk * 48) >> 2, e = r & 3;
+  xT[(size_t)half * BP * D + ((size_t)((fbk * 12 + nn) * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
 }
 
 __global__ void tiled_zero_kernel(float* p, int n) {
@@ -262,14 +265,81 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 }
 
 // ---- grad_W and the SGD update of one chunk, in place.  blockIdx = tile*4 + fb; wavefront w owns label rows 16w..16w+15
-//      of the tile and features 192fb.. (12 blocks of 16).  A^T[f][l] = sum_b X^T[f][b] G[l][b]; a lane ends up with four
-//      consecutive features of one label row.
+//      of the tile and features 192fb.. (12 blocks of 16).  A^T[f][l] = sum_b X^T[f][b] G[l][b].  The rows of a feature
+//      block are permuted (row 4kg+e of block nn is feature 192fb + 48kg + 4nn + e, see tiled_prep_x_kernel) so that a
+//      lane ends up with 48 consecutive features of one label row and moves them 16 at a time.
 //        bf16 weights : a = bf16(A); t = w - lr*a; RTN: bf16(t);  SR: bits(t) + (philox(seed, l*768+f) & 0xFFFF), clear 16 bits
 //        e4m3 weights : t = w - lr*A;          RTN: e4m3(t); SR: add 20 bits, clear, same cast.  The cast is torch's (NaN above
 //                       464; simulated FP8, chunked_fp8xmc_clf.py:116) or saturating at +-448 (true FP8, fuse_kernel.py:35).
 //        head-Kahan (e4m3 weights, rows below num_head; fuse_kernel.py:202-262): t = (w + k) - lr*A, W' = round(t),
 //                       k' = ((k + w) - W') - lr*A stored as bf16 (kahan_type 1) or e5m2 (2); rows behind the head take
 //                       their random offsets from (row - num_head), as the reference's call on the sliced tensors does
+// Four consecutive features of one row: old weights (bf16: two dwords, e4m3: one) and compensation terms in, new ones out.
+template <int WT, int MODE>
+__device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const unsigned* kraw, bool head, int kahan_type, float lr,
+                                          unsigned off0, unsigned seed, int saturate, unsigned* wout, unsigned* kout) {
+  float wv4[4];
+  if (WT == W_BF16) {
+    wv4[0] = bf16_from_bits((unsigned short)(wraw[0] & 0xffffu)); wv4[1] = bf16_from_bits((unsigned short)(wraw[0] >> 16));
+    wv4[2] = bf16_from_bits((unsigned short)(wraw[1] & 0xffffu)); wv4[3] = bf16_from_bits((unsigned short)(wraw[1] >> 16));
+  } else {
+    floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wraw[0], false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wraw[0], true);
+    wv4[0] = w01.x; wv4[1] = w01.y; wv4[2] = w23.x; wv4[3] = w23.y;
+  }
+  float kv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (head) {
+    if (kahan_type == 1) {
+      kv[0] = bf16_from_bits((unsigned short)(kraw[0] & 0xffffu)); kv[1] = bf16_from_bits((unsigned short)(kraw[0] >> 16));
+      kv[2] = bf16_from_bits((unsigned short)(kraw[1] & 0xffffu)); kv[3] = bf16_from_bits((unsigned short)(kraw[1] >> 16));
+    } else {
+      floatx2 k01 = __builtin_amdgcn_cvt_pk_f32_bf8((int)kraw[0], false), k23 = __builtin_amdgcn_cvt_pk_f32_bf8((int)kraw[0], true);
+      kv[0] = k01.x; kv[1] = k01.y; kv[2] = k23.x; kv[3] = k23.y;
+    }
+  }
+  float t[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const float g = WT == W_BF16 ? bf16_rt(a[e]) : a[e];
+    t[e] = __builtin_fmaf(-lr, g, head ? wv4[e] + kv[e] : wv4[e]);
+    if (MODE == ROUND_SR_PHILOX) {
+      const unsigned r = philox_word0(off0 + (unsigned)e, seed, 0u);
+      const unsigned mask = WT == W_BF16 ? 0xFFFFu : 0xFFFFFu;
+      t[e] = __uint_as_float((__float_as_uint(t[e]) + (r & mask)) & ~mask);
+    }
+  }
+  if (WT == W_BF16) {
+    wout[0] = (unsigned)bf16_bits(t[0]) | ((unsigned)bf16_bits(t[1]) << 16);
+    wout[1] = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
+  } else {
+    if (saturate) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) t[e] = clamp448(t[e]);
+    }
+    int packed = 0;   // without the clamp: torch's cast gives NaN above 464 and so does the converter
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
+    wout[0] = (unsigned)packed;
+    if (head) {
+      floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, true);
+      const float wn[4] = {n01.x, n01.y, n23.x, n23.y};
+      float kn[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) kn[e] = __builtin_fmaf(-lr, a[e], (kv[e] + wv4[e]) - wn[e]);
+      if (kahan_type == 1) {
+        kout[0] = (unsigned)bf16_bits(kn[0]) | ((unsigned)bf16_bits(kn[1]) << 16);
+        kout[1] = (unsigned)bf16_bits(kn[2]) | ((unsigned)bf16_bits(kn[3]) << 16);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
+        int pk = 0;
+        pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
+        pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
+        kout[0] = (unsigned)pk;
+      }
+    }
+  }
+}
+
 template <int WT, int MODE>
 __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, size_t g_half_stride,
                                                            int halves, const unsigned short* xT, float lr, unsigned seed,
@@ -277,99 +347,70 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, tile = blockIdx.x >> 2;
   const int row = tile * TL + 16 * wv + l16;
+  const bool live = row < rows;
+  const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
+  const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
   bf16x8 gf[T_HALVES][4];
 #pragma unroll
   for (int hh = 0; hh < T_HALVES; hh++)
 #pragma unroll
     for (int ks = 0; ks < 4; ks++)
       gf[hh][ks] = hh < halves ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
-#pragma unroll 2
-  for (int nn = 0; nn < 12; nn++) {
-    const int f = 192 * fb + 16 * nn;
-    floatx4 a = {0.f, 0.f, 0.f, 0.f};
+  constexpr int WDW = WT == W_BF16 ? 8 : 4;   // dwords of 16 weights
+#pragma unroll 1
+  for (int c = 0; c < 3; c++) {               // 16 consecutive features of this lane's row at a time
+    const int col0 = 192 * fb + 48 * kg + 16 * c;
+    const size_t idx = (size_t)row * D + col0;
+    unsigned wr[WDW], wo[WDW], kr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, ko[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int hh = 0; hh < T_HALVES; hh++) {
-      if (hh < halves) {
+    for (int q = 0; q < WDW; q++) { wr[q] = 0; wo[q] = 0; }
+    if (live) {
+      const intx4* src = (const intx4*)((const unsigned char*)w + idx * (WT == W_BF16 ? 2 : 1));
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-          const bf16x8 xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((f >> 4) * (BP / 32) + ks) * 64 + lane) * 8);
-          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
+      for (int q = 0; q < WDW / 4; q++) {
+        const intx4 v = src[q];
+        wr[4 * q] = (unsigned)v.x; wr[4 * q + 1] = (unsigned)v.y; wr[4 * q + 2] = (unsigned)v.z; wr[4 * q + 3] = (unsigned)v.w;
+      }
+      if (head) {
+        const int kdw = kahan_type == 1 ? 8 : 4;
+        const intx4* ksrc = (const intx4*)((const unsigned char*)kahan + idx * (kahan_type == 1 ? 2 : 1));
+        const intx4 v0 = ksrc[0];
+        kr[0] = (unsigned)v0.x; kr[1] = (unsigned)v0.y; kr[2] = (unsigned)v0.z; kr[3] = (unsigned)v0.w;
+        if (kdw == 8) {
+          const intx4 v1 = ksrc[1];
+          kr[4] = (unsigned)v1.x; kr[5] = (unsigned)v1.y; kr[6] = (unsigned)v1.z; kr[7] = (unsigned)v1.w;
         }
       }
     }
-    // a[e] = A[label row][feature f + 4kg + e]
-    if (row < rows) {
-      const int col = f + 4 * kg;
-      const size_t idx = (size_t)row * D + col;
-      float wv4[4];
-      if (WT == W_BF16) {
-        const uint2 raw = *(const uint2*)((const unsigned short*)w + idx);
-        wv4[0] = bf16_from_bits((unsigned short)(raw.x & 0xffffu)); wv4[1] = bf16_from_bits((unsigned short)(raw.x >> 16));
-        wv4[2] = bf16_from_bits((unsigned short)(raw.y & 0xffffu)); wv4[3] = bf16_from_bits((unsigned short)(raw.y >> 16));
-      } else {
-        const int raw = *(const int*)((const unsigned char*)w + idx);
-        floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8(raw, true);
-        wv4[0] = w01.x; wv4[1] = w01.y; wv4[2] = w23.x; wv4[3] = w23.y;
-      }
-      const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
-      const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
-      float kv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (head) {
-        if (kahan_type == 1) {
-          const uint2 raw = *(const uint2*)((const unsigned short*)kahan + idx);
-          kv[0] = bf16_from_bits((unsigned short)(raw.x & 0xffffu)); kv[1] = bf16_from_bits((unsigned short)(raw.x >> 16));
-          kv[2] = bf16_from_bits((unsigned short)(raw.y & 0xffffu)); kv[3] = bf16_from_bits((unsigned short)(raw.y >> 16));
-        } else {
-          const int raw = *(const int*)((const unsigned char*)kahan + idx);
-          floatx2 k01 = __builtin_amdgcn_cvt_pk_f32_bf8(raw, false), k23 = __builtin_amdgcn_cvt_pk_f32_bf8(raw, true);
-          kv[0] = k01.x; kv[1] = k01.y; kv[2] = k23.x; kv[3] = k23.y;
-        }
-      }
-      float t[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const float g = WT == W_BF16 ? bf16_rt(a[e]) : a[e];
-        t[e] = __builtin_fmaf(-lr, g, head ? wv4[e] + kv[e] : wv4[e]);
-        if (MODE == ROUND_SR_PHILOX) {
-          const unsigned r = philox_word0((unsigned)orow * (unsigned)D + (unsigned)(col + e), seed, 0u);
-          const unsigned mask = WT == W_BF16 ? 0xFFFFu : 0xFFFFFu;
-          t[e] = __uint_as_float((__float_as_uint(t[e]) + (r & mask)) & ~mask);
-        }
-      }
-      if (WT == W_BF16) {
-        uint2 o;
-        o.x = (unsigned)bf16_bits(t[0]) | ((unsigned)bf16_bits(t[1]) << 16);
-        o.y = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
-        *(uint2*)((unsigned short*)w + idx) = o;
-      } else {
-        if (saturate) {
+    for (int q = 0; q < 4; q++) {
+      const int nn = 4 * c + q;
+      floatx4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int e = 0; e < 4; e++) t[e] = clamp448(t[e]);
-        }
-        int packed = 0;   // without the clamp: torch's cast gives NaN above 464 and so does the converter
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
-        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
-        *(int*)((unsigned char*)w + idx) = packed;
-        if (head) {
-          floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, true);
-          const float wn[4] = {n01.x, n01.y, n23.x, n23.y};
-          float kn[4];
+      for (int hh = 0; hh < T_HALVES; hh++) {
+        if (hh < halves) {
 #pragma unroll
-          for (int e = 0; e < 4; e++) kn[e] = __builtin_fmaf(-lr, a[e], (kv[e] + wv4[e]) - wn[e]);
-          if (kahan_type == 1) {
-            uint2 o;
-            o.x = (unsigned)bf16_bits(kn[0]) | ((unsigned)bf16_bits(kn[1]) << 16);
-            o.y = (unsigned)bf16_bits(kn[2]) | ((unsigned)bf16_bits(kn[3]) << 16);
-            *(uint2*)((unsigned short*)kahan + idx) = o;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
-            int pk = 0;
-            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
-            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
-            *(int*)((unsigned char*)kahan + idx) = pk;
+          for (int ks = 0; ks < 4; ks++) {
+            const bf16x8 xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((fb * 12 + nn) * (BP / 32) + ks) * 64 + lane) * 8);
+            a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
           }
         }
+      }
+      // a[e] = A[label row][feature col0 + 4q + e]
+      if (live) {
+        const int wq = WT == W_BF16 ? 2 * q : q, kq = kahan_type == 1 ? 2 * q : q;
+        t_update4<WT, MODE>(a, wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q), seed,
+                            saturate, wo + wq, ko + kq);
+      }
+    }
+    if (live) {
+      intx4* dst = (intx4*)((unsigned char*)w + idx * (WT == W_BF16 ? 2 : 1));
+#pragma unroll
+      for (int q = 0; q < WDW / 4; q++) dst[q] = intx4{(int)wo[4 * q], (int)wo[4 * q + 1], (int)wo[4 * q + 2], (int)wo[4 * q + 3]};
+      if (head) {
+        intx4* kdst = (intx4*)((unsigned char*)kahan + idx * (kahan_type == 1 ? 2 : 1));
+        kdst[0] = intx4{(int)ko[0], (int)ko[1], (int)ko[2], (int)ko[3]};
+        if (kahan_type == 1) kdst[1] = intx4{(int)ko[4], (int)ko[5], (int)ko[6], (int)ko[7]};
       }
     }
   }
