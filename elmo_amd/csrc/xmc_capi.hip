@@ -30,6 +30,10 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
     (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
+    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
   }
   return cached[dev];
 }
@@ -236,8 +240,8 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
   const size_t halves = ((size_t)max_batch + BP - 1) / BP;
-  // per batch half G in both orientations; tile_ptr (padded to 64 entries); one loss share per tile
-  return TW_G + halves * 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 4 + 255) / 256 * 256;
+  // per batch half G in both orientations; tile_ptr (padded to 64 entries); two loss shares per tile
+  return TW_G + halves * 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 8 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
@@ -280,7 +284,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   unsigned short* glb = (unsigned short*)(ws + TW_G);
   unsigned short* gbl = glb + (size_t)rows_pad * BP;
   int* tile_ptr = (int*)(glb + halves * g_half);
-  float* loss_part = (float*)(tile_ptr + (num_tiles + 1 + 63) / 64 * 64);   // one share per tile
+  float* loss_part = (float*)(tile_ptr + (num_tiles + 1 + 63) / 64 * 64);   // one share per sub-tile of 32 rows
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
@@ -289,7 +293,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
   tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT);
   tiled_zero_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>(gx_total, halves * BP * D);
-  if (loss_out) tiled_zero_kernel<<<(num_tiles + 255) / 256, 256, 0, stream>>>(loss_part, num_tiles);
+  if (loss_out) tiled_zero_kernel<<<(2 * num_tiles + 255) / 256, 256, 0, stream>>>(loss_part, 2 * num_tiles);
   for (int c = 0; c < num_chunks; c++) {
     void* w = chunk_ptrs[c];
     const int rows = c == num_chunks - 1 ? rows_last_chunk : rows_per_chunk;
@@ -302,22 +306,24 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     range = (range + TL - 1) / TL * TL;
     const int splits = (rp + range - 1) / range;
     const int* tp = tile_ptr + c * tiles_per_chunk;
-    float* lp = loss_part + c * tiles_per_chunk;
+    float* lp = loss_part + 2 * c * tiles_per_chunk;
     for (int hh = 0; hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
       unsigned short* gb = gbl + hh * g_half;
       const unsigned short* xh = xb + (size_t)hh * BP * D;
       const unsigned brow0 = (unsigned)(hh * BP);
+      const int nsub = 2 * tiles;                                   // sub-tiles of 32 label rows
+      const int lgrid = nsub < di.cus ? nsub : di.cus;              // persistent: one workgroup per compute unit
       if (weight_type == W_BF16) {
-        if (loss_out) tiled_logits_kernel<W_BF16, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        else tiled_logits_kernel<W_BF16, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       } else {
-        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        else tiled_logits_kernel<W_E4M3, false><<<tiles, 256, 0, stream>>>(w, rows, rows_pad, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       }
-      tiled_reduce_kernel<<<96, 256, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
+      tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
     if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
@@ -328,7 +334,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     }
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
-  if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, num_tiles, loss_out);
+  if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, 2 * num_tiles, loss_out);
   return launch_status();
 }
 

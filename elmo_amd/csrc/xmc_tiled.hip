@@ -8,6 +8,7 @@
 // not the headline path: the kernels take their operands straight from global memory (L2) in MFMA operand order and
 // stage only the one operand that needs a transposition (W in grad_X) through LDS.
 #include "xmc_common.h"
+#include <type_traits>
 
 namespace xmc {
 
@@ -73,91 +74,169 @@ __global__ void tiled_zero_kernel(float* p, int n) {
   if (i < n) p[i] = 0.f;
 }
 
-// ---- logits, sigmoid minus targets.  One workgroup per 64 label rows, wavefront w takes rows 16w..16w+15 against the
-//      whole (padded) batch.  Writes G[l][b] and G^T[b][l]; rows beyond the chunk are written as zeros.
-//      LOSS: also the workgroup's share of the summed binary cross entropy of the bf16 logits z against the targets,
+// ---- logits, sigmoid minus targets.  Persistent workgroups of 8 wavefronts; wavefront v keeps the X operand of batch
+//      rows 16v..16v+15 of this half in registers (96 of them) for the whole launch.  The label rows stream through LDS
+//      in sub-tiles of 32 rows (coalesced 16-byte loads into registers one sub-tile ahead, then LDS, two buffers, one
+//      barrier per sub-tile); every wavefront multiplies the sub-tile with its batch rows.  Writes G[l][b] row-major
+//      and G^T in the operand order of the grad_X kernel; rows beyond the chunk are written as zeros.
+//      LOSS: also the sub-tile's share of the summed binary cross entropy of the bf16 logits z against the targets,
 //      sum over labels and batch rows of max(z, 0) - [positive] z + log(1 + exp(-|z|)), the quantity that
-//      _compute_loss of the reference is written to return (chunked.py:57-72), in fp32 and stored per workgroup for a
+//      _compute_loss of the reference is written to return (chunked.py:57-72), in fp32 and added per sub-tile for a
 //      fixed-order sum.
+constexpr int TLG_ROWS = 32;
+template <int WT> struct TlgGeom {
+  static constexpr int ROWB = WT == W_BF16 ? D * 2 : D;                 // bytes of one weight row
+  static constexpr int STRIDE = ROWB + 16;                               // LDS row stride
+  static constexpr int SLOTS = STRIDE / 16;                              // 16-byte slots per LDS row, the last one padding
+  static constexpr int PIECES = (TLG_ROWS * STRIDE + 1023) / 1024;       // wave-wide direct-to-LDS loads per sub-tile (49 or 25)
+  static constexpr int BUF = PIECES * 1024;                              // bytes of one LDS buffer
+  static constexpr int PER_WAVE = (PIECES + 7) / 8;                      // loads of wavefront 0 (7 or 4); the others issue at
+  static constexpr int PER_WAVE_MIN = PIECES / 8;                        // least this many (6 or 3)
+  static constexpr int LDS = 3 * BUF + 64;                               // three buffers and eight partial sums of the loss
+};
+
+// 16 bytes per lane from global memory straight into LDS at byte offset ldsoff + 16*lane (wave-uniform offset).  Inline
+// assembly: the compiler neither orders later LDS accesses behind it nor waits for it; completion is enforced by hand.
+__device__ __forceinline__ void t_lds_load16(const unsigned char* g, unsigned ldsoff_) {
+  const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsoff), "v"(g) : "memory", "m0");
+}
+
+// Vector memory operations retire in order.  Per sub-tile a wavefront issues its loads of the sub-tile two steps ahead
+// (always, past the end they fetch the last sub-tile again into a buffer nobody reads, so that the count is the same in
+// every step) and then ten stores of G.  The wait at the top of a step leaves in flight what was issued after the
+// loads of the sub-tile it is about to read.
 template <int WT, bool LOSS>
-__global__ __launch_bounds__(256) void tiled_logits_kernel(const void* w, int rows, int rows_pad, const unsigned short* xb,
-                                                           const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
-                                                           unsigned short* glb, unsigned short* gbl, int batch, unsigned brow0,
-                                                           float* loss_part) {
-  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int r0 = blockIdx.x * TL + 16 * wv;
-  const int lrow = min(r0 + l16, rows - 1);
-  floatx4 acc[8];
+__global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int rows, int nsub, const unsigned short* xb,
+                                                              const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
+                                                              unsigned short* glb, unsigned short* gbl, int batch, unsigned brow0,
+                                                              float* loss_part) {
+  typedef TlgGeom<WT> G;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tlg_lds[];
+  __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tlg_lds;
+  // no static LDS in this kernel: the direct-to-LDS loads address LDS from byte 0
+  __attribute__((address_space(3))) float* wsum = (__attribute__((address_space(3))) float*)(lds + 3 * G::BUF);
+  const int tid = threadIdx.x, v = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  // the sorted keys and the tile ranges were written by earlier launches: read them through the scalar (constant) path,
+  // so that no vector-memory wait of this loop covers them
+  const __attribute__((address_space(4))) unsigned* ckeys = (const __attribute__((address_space(4))) unsigned*)keys;
+  const __attribute__((address_space(4))) int* ctile_ptr = (const __attribute__((address_space(4))) int*)tile_ptr;
+  // source row and byte offset within the row of this lane's slot in pieces v, v+8, ..
+  int prow[G::PER_WAVE], pcol[G::PER_WAVE];
 #pragma unroll
-  for (int nb = 0; nb < 8; nb++) acc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-  for (int ks = 0; ks < D / 32; ks++) {
-    const bf16x8 a = t_load_w8<WT>(w, (size_t)lrow * D + 32 * ks + 8 * kg);
-#pragma unroll
-    for (int nb = 0; nb < 8; nb++) {
-      const bf16x8 b = *(const bf16x8*)(xb + ((size_t)(nb * (D / 32) + ks) * 64 + lane) * 8);
-      acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nb], 0, 0, 0);
-    }
+  for (int s = 0; s < G::PER_WAVE; s++) {
+    const int slot = (v + 8 * s) * 64 + lane;
+    prow[s] = min(slot / G::SLOTS, TLG_ROWS - 1);
+    pcol[s] = min(slot - (slot / G::SLOTS) * G::SLOTS, G::SLOTS - 2) * 16;
   }
-  // acc[nb][e] = Z[label r0 + 4kg + e][batch 16nb + l16]
-  const float nlog2e = -1.44269504088896340736f;
-  float sg[8][4];
-  float lsum = 0.f;
+  auto issue_sub = [&](int st, int buf) {
+    const int s0 = min(st, nsub - 1) * TLG_ROWS;
 #pragma unroll
-  for (int nb = 0; nb < 8; nb++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      float zf = bf16_rt(acc[nb][e]);
-      const float ex = __builtin_amdgcn_exp2f(zf * nlog2e);   // exp(-z)
-      sg[nb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + ex));
-      if (LOSS) {
-        acc[nb][e] = zf;   // kept for the positives below
-        if (r0 + 4 * kg + e < rows && (int)brow0 + 16 * nb + l16 < batch)
-          lsum += __builtin_fmaxf(zf, 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf) * 1.44269504088896340736f));
+    for (int s = 0; s < G::PER_WAVE; s++) {
+      if (v + 8 * s < G::PIECES) {
+        const int lr = min(s0 + prow[s], rows - 1);
+        t_lds_load16((const unsigned char*)w + (size_t)lr * G::ROWB + pcol[s], (unsigned)(buf * G::BUF + (v + 8 * s) * 1024));
       }
     }
-  // positives of this tile (set semantics: a repeated key counts once)
-  const int p0 = tile_ptr[blockIdx.x], p1 = tile_ptr[blockIdx.x + 1];
-  const unsigned lbase = label0_chunk + (unsigned)(r0 + 4 * kg);
-  for (int e = p0; e < p1; e++) {
-    const unsigned key = keys[e];
-    const unsigned prev = e > 0 ? keys[e - 1] : ~key;
-    const unsigned l = (key >> 8) - lbase;
-    const unsigned b = (key & 255u) - brow0;   // batch row within this half
-    if (prev != key && l < 4u && b < (unsigned)BP && (b & 15u) == (unsigned)l16) {
+  };
+  const float nlog2e = -1.44269504088896340736f;
+  const int gs = (int)gridDim.x;
+  issue_sub(blockIdx.x, 0);
+  issue_sub(blockIdx.x + gs, 1);
+  // the X operand of this wavefront's batch rows, behind the first two sub-tiles in the memory pipeline
+  bf16x8 xr[D / 32];
 #pragma unroll
-      for (int nb = 0; nb < 8; nb++)
+  for (int ks = 0; ks < D / 32; ks++) xr[ks] = *(const bf16x8*)(xb + ((size_t)(v * (D / 32) + ks) * 64 + lane) * 8);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // from here on the loop counts its own operations: nothing is in flight
+  int it = 0, b0 = 0, b2 = 2;   // it % 3, (it + 2) % 3
+  for (int st = blockIdx.x; st < nsub; st += gs, it++) {
+    // younger than the loads of this sub-tile: the loads of the next one and the stores of up to two steps
+    if (it == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN) : "memory");
+    else if (it == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 10) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 20) : "memory");
+    // range of positives of the enclosing 64-row tile: asked for here, needed after the MFMAs
+    const int p0 = ctile_ptr[st >> 1], p1 = ctile_ptr[(st >> 1) + 1];
+    __syncthreads();
+    issue_sub(st + 2 * gs, b2);
+    const int buf = b0;
+    b0 = b0 == 2 ? 0 : b0 + 1;
+    b2 = b2 == 2 ? 0 : b2 + 1;
+    floatx4 acc[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    const unsigned abase = (unsigned)(buf * G::BUF + l16 * G::STRIDE + kg * (WT == W_BF16 ? 16 : 8));
+    // the LDS reads run three K steps ahead of the MFMAs (everything unrolled: xr must stay in registers)
+    typedef typename std::conditional<WT == W_BF16, bf16x8, intx2>::type araw_t;
+    araw_t araw[4][2];
+    auto rd = [&](int ks, int lb) {
+      if (WT == W_BF16) return *(const __attribute__((address_space(3))) araw_t*)(lds + abase + lb * 16 * G::STRIDE + ks * 64);
+      else return *(const __attribute__((address_space(3))) araw_t*)(lds + abase + lb * 16 * G::STRIDE + ks * 32);
+    };
 #pragma unroll
-        for (int q4 = 0; q4 < 4; q4++)
-          if ((b >> 4) == (unsigned)nb && l == (unsigned)q4) {
-            sg[nb][q4] = bf16_rt(sg[nb][q4] - 1.0f);
-            if (LOSS && r0 + 4 * kg + q4 < rows) lsum -= acc[nb][q4];
-          }
+    for (int ks = 0; ks < 3; ks++) { araw[ks][0] = rd(ks, 0); araw[ks][1] = rd(ks, 1); }
+#pragma unroll
+    for (int ks = 0; ks < D / 32; ks++) {
+      if (ks + 3 < D / 32) { araw[(ks + 3) & 3][0] = rd(ks + 3, 0); araw[(ks + 3) & 3][1] = rd(ks + 3, 1); }
+      __builtin_amdgcn_sched_barrier(0);   // keep the reads ahead of the MFMAs that do not need them yet
+#pragma unroll
+      for (int lb = 0; lb < 2; lb++) {
+        bf16x8 a;
+        if constexpr (WT == W_BF16) a = araw[ks & 3][lb];
+        else a = t_fp8x8_to_bf16x8(araw[ks & 3][lb]);
+        acc[lb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xr[ks], acc[lb], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // acc[lb][e] = Z[label 32 st + 16 lb + 4kg + e][batch 16v + l16]
+    float lsum = 0.f;
+#pragma unroll
+    for (int lb = 0; lb < 2; lb++) {
+      const int r0 = st * TLG_ROWS + 16 * lb;
+      float sg[4], zf[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        zf[e] = bf16_rt(acc[lb][e]);
+        sg[e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf[e] * nlog2e)));
+        if (LOSS && r0 + 4 * kg + e < rows && (int)brow0 + 16 * v + l16 < batch)
+          lsum += __builtin_fmaxf(zf[e], 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf[e]) * 1.44269504088896340736f));
+      }
+      // positives of the enclosing 64-row tile (set semantics: a repeated key counts once)
+      const unsigned lbase = label0_chunk + (unsigned)(r0 + 4 * kg);
+      for (int e = p0; e < p1; e++) {
+        const unsigned key = ckeys[e];
+        const unsigned prev = e > 0 ? ckeys[e - 1] : ~key;
+        const unsigned l = (key >> 8) - lbase;
+        const unsigned b = (key & 255u) - brow0;   // batch row within this half
+        if (prev != key && l < 4u && b == (unsigned)(16 * v + l16)) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; q4++)
+            if (l == (unsigned)q4) {
+              sg[q4] = bf16_rt(sg[q4] - 1.0f);
+              if (LOSS && r0 + 4 * kg + q4 < rows) lsum -= zf[q4];
+            }
+        }
+      }
+      unsigned short sb[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[e]) : (unsigned short)0;
+      const int b = 16 * v + l16;
+      uint2 o;
+      o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
+      o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
+      // G^T in operand order for grad_X: block (label / 32, batch block) of 16 batch rows x 32 labels
+      *(uint2*)(gbl + ((size_t)(st * 8 + v) * 64 + l16 + 16 * (2 * lb + (kg >> 1))) * 8 + 4 * (kg & 1)) = o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
+
+    }
+    if (LOSS) {
+      // lanes of a wavefront, then the eight wavefronts, in a fixed order; the halves of the batch run one after the other
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
+      if (lane == 0) wsum[v] = lsum;
+      __syncthreads();
+      if (tid == 0) loss_part[st] += ((wsum[0] + wsum[1]) + (wsum[2] + wsum[3])) + ((wsum[4] + wsum[5]) + (wsum[6] + wsum[7]));
     }
   }
-  if (LOSS) {
-    // lanes of a wavefront, then the four wavefronts, in a fixed order
-    __shared__ float wsum[4];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
-    if (lane == 0) wsum[wv] = lsum;
-    __syncthreads();
-    if (tid == 0) loss_part[blockIdx.x] += (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);   // the halves run one after the other
-  }
-#pragma unroll
-  for (int nb = 0; nb < 8; nb++) {
-    unsigned short sb[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[nb][e]) : (unsigned short)0;
-    const int b = 16 * nb + l16;
-    uint2 o;
-    o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
-    o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
-    // G^T in operand order for grad_X: block (label / 32, nb) of 16 batch rows x 32 labels
-    *(uint2*)(gbl + ((size_t)((blockIdx.x * 2 + (wv >> 1)) * 8 + nb) * 64 + l16 + 16 * (2 * (wv & 1) + (kg >> 1))) * 8 + 4 * (kg & 1)) = o;
-#pragma unroll
-    for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
-  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last loads still target LDS
 }
 
 // sum of the per-workgroup loss shares in a fixed order (double precision), one workgroup
@@ -191,15 +270,40 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lbeg = split * range, lend = min(lbeg + range, bound);   // bound: this chunk's rows rounded up to a tile
+  // The operands of step l0 + 32 are loaded into registers while step l0 computes.
+  constexpr int NW = WT == W_BF16 ? 3 : 2;   // 16-byte pieces of W per lane and step
+  intx4 wraw[NW], wnext[NW];
+  bf16x8 ga[8], gnext[8];
+  auto load_step = [&](int l0, intx4* wr, bf16x8* g) {
+#pragma unroll
+    for (int s = 0; s < NW; s++) {
+      const int c = lane + 64 * s;
+      if (WT == W_BF16) {
+        const int row = c / 6, c16 = c - row * 6;
+        const int lr = min(l0 + row, rows - 1);
+        wr[s] = *(const intx4*)((const unsigned short*)w + (size_t)lr * D + f0 + 8 * c16);
+      } else {
+        const int cc = min(c, 95), row = cc / 3, c16 = cc - row * 3;
+        const int lr = min(l0 + row, rows - 1);
+        wr[s] = *(const intx4*)((const unsigned char*)w + (size_t)lr * D + f0 + 16 * c16);
+      }
+    }
+#pragma unroll
+    for (int mb = 0; mb < 8; mb++) g[mb] = *(const bf16x8*)(gbl + ((size_t)((l0 >> 5) * 8 + mb) * 64 + lane) * 8);
+  };
+  if (lbeg < lend) load_step(lbeg, wnext, gnext);
   for (int l0 = lbeg; l0 < lend; l0 += 32) {
-    // W[l0..l0+31][f0..f0+47] -> LDS as bf16, row stride T_WS2
+#pragma unroll
+    for (int s = 0; s < NW; s++) wraw[s] = wnext[s];
+#pragma unroll
+    for (int mb = 0; mb < 8; mb++) ga[mb] = gnext[mb];
+    if (l0 + 32 < lend) load_step(l0 + 32, wnext, gnext);
+    // W[l0..l0+31][f0..f0+47] -> LDS as bf16, row stride T_WS2 (the wavefront's own block: no barrier needed)
     if (WT == W_BF16) {
 #pragma unroll
       for (int s = 0; s < 3; s++) {
         const int c = lane + 64 * s, row = c / 6, c16 = c - row * 6;
-        const int lr = min(l0 + row, rows - 1);
-        const intx4 v = *(const intx4*)((const unsigned short*)w + (size_t)lr * D + f0 + 8 * c16);
-        *(__attribute__((address_space(3))) intx4*)(lw + row * T_WS2 + c16 * 16) = v;
+        *(__attribute__((address_space(3))) intx4*)(lw + row * T_WS2 + c16 * 16) = wraw[s];
       }
     } else {
 #pragma unroll
@@ -207,17 +311,12 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
         const int c = lane + 64 * s;
         if (c < 96) {
           const int row = c / 3, c16 = c - row * 3;
-          const int lr = min(l0 + row, rows - 1);
-          const intx4 v = *(const intx4*)((const unsigned char*)w + (size_t)lr * D + f0 + 16 * c16);
-          const bf16x8 lo = t_fp8x8_to_bf16x8(intx2{v.x, v.y}), hi = t_fp8x8_to_bf16x8(intx2{v.z, v.w});
+          const bf16x8 lo = t_fp8x8_to_bf16x8(intx2{wraw[s].x, wraw[s].y}), hi = t_fp8x8_to_bf16x8(intx2{wraw[s].z, wraw[s].w});
           *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32) = lo;
           *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32 + 16) = hi;
         }
       }
     }
-    bf16x8 ga[8];
-#pragma unroll
-    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const bf16x8*)(gbl + ((size_t)((l0 >> 5) * 8 + mb) * 64 + lane) * 8);
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
@@ -241,11 +340,20 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
 
 // sum of the partials of one chunk in a fixed order; bf16 weights: the chunk's contribution is rounded to bf16 before it
 // is added to the fp32 total (chunked.py:116)
-__global__ __launch_bounds__(256) void tiled_reduce_kernel(const floatx4* partial, int splits, int round_bf16, float* gx_total) {
-  const int slot = blockIdx.x >> 2, fb = blockIdx.x & 3;
-  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+__global__ __launch_bounds__(64) void tiled_reduce_kernel(const floatx4* partial, int splits, int round_bf16, float* gx_total) {
+  // 384 workgroups of one wavefront: (slot, fb, wavefront of the grad_X kernel's layout); eight loads in flight
+  const int slot = blockIdx.x >> 4, fb = (blockIdx.x >> 2) & 3, wv = blockIdx.x & 3;
+  const int lane = threadIdx.x, tid = wv * 64 + lane, l16 = lane & 15, kg = lane >> 4;
   floatx4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int sp = 0; sp < splits; sp++) s += partial[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
+  int sp = 0;
+  for (; sp + 8 <= splits; sp += 8) {
+    floatx4 v[8];
+#pragma unroll
+    for (int x = 0; x < 8; x++) v[x] = partial[(((size_t)(sp + x) * 4 + fb) * 24 + slot) * 256 + tid];
+#pragma unroll
+    for (int x = 0; x < 8; x++) s += v[x];
+  }
+  for (; sp < splits; sp++) s += partial[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
   const int mb = slot / 3, nn = slot - mb * 3;
   const int col = 192 * fb + 48 * wv + 16 * nn + l16;
 #pragma unroll
