@@ -42,6 +42,11 @@ def load():
     lib.xmc_tiled_step.restype = i32
     lib.xmc_tiled_step.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32, vp, i32, i32, vp, i32, f32,
                                    ctypes.POINTER(ctypes.c_uint32), i32, i32, i32, vp, i32, i32, vp, vp, vp, vp, sz, vp]
+    lib.xmc_topk_scratch_bytes.restype = sz
+    lib.xmc_topk_scratch_bytes.argtypes = [i32]
+    lib.xmc_fp8_forward_topk.restype = i32
+    lib.xmc_fp8_forward_topk.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp, vp,
+                                         vp, sz, vp, sz, vp]
     lib.xmc_select_step_kernel.restype = i32
     lib.xmc_select_step_kernel.argtypes = [i32]
     lib.xmc_copy_probe.restype = i32

@@ -4,6 +4,7 @@
 #include "xmc_fp8_step.hip"
 #include "xmc_fp8_quad.hip"
 #include "xmc_tiled.hip"
+#include "xmc_topk.hip"
 #include <stdlib.h>
 
 using namespace xmc;
@@ -226,6 +227,49 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
     fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
                                                        scale_w * scale_x, (unsigned short*)out_bf16, out_stride,
                                                        (long long)c * rows_per_chunk, num_labels, batch);
+  return launch_status();
+}
+
+size_t xmc_topk_scratch_bytes(int rows_per_chunk) {
+  if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return 0;
+  // logits of one chunk [128][rows] bf16, then the running lists: values [128][128] bf16, label ids [128][128] int32
+  return ((size_t)BP * rows_per_chunk * 2 + 255) / 256 * 256 + (size_t)BP * TOPK_MAX * 2 + (size_t)BP * TOPK_MAX * 4;
+}
+
+int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                         int features, float scale_w, float scale_x, long long num_labels, int k, void* out_val_bf16,
+                         int32_t* out_idx, void* workspace, size_t workspace_bytes, void* scratch, size_t scratch_bytes,
+                         void* stream_) {
+  int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
+  if (st != XMC_OK) return st;
+  if (!out_val_bf16 || !out_idx || !scratch) return XMC_ERR_NULL;
+  if (((uintptr_t)scratch & 255) != 0) return XMC_ERR_ALIGN;
+  if (scratch_bytes < xmc_topk_scratch_bytes(rows_per_chunk)) return XMC_ERR_WORKSPACE;
+  if (num_labels <= 0 || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
+  if (k <= 0 || k > TOPK_MAX || k > num_labels) return XMC_ERR_SHAPE;
+  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  unsigned char* ws = (unsigned char*)workspace;
+  unsigned short* zbuf = (unsigned short*)scratch;
+  unsigned short* run_val = (unsigned short*)((unsigned char*)scratch + ((size_t)BP * rows_per_chunk * 2 + 255) / 256 * 256);
+  int* run_idx = (int*)(run_val + (size_t)BP * TOPK_MAX);
+  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
+                                                              (unsigned short*)(ws + WS_XT));
+  const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
+  const int grid = tiles_per_chunk < 4 * di.cus ? tiles_per_chunk : 4 * di.cus;
+  int have = 0;
+  for (int c = 0; c < num_chunks; c++) {
+    const long long base = (long long)c * rows_per_chunk;
+    if (base >= num_labels) break;
+    const int n = (int)(num_labels - base < rows_per_chunk ? num_labels - base : rows_per_chunk);   // padding rows are dropped
+    fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
+                                                       scale_w * scale_x, zbuf, rows_per_chunk, 0, n, batch);
+    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, rows_per_chunk, n, (int)base, k, have, run_val, run_idx);
+    have = have + n < k ? have + n : k;
+  }
+  topk_finish_kernel<<<(batch * k + 255) / 256, 256, 0, stream>>>(run_val, run_idx, batch, k, (unsigned short*)out_val_bf16, out_idx);
   return launch_status();
 }
 

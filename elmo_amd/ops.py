@@ -94,6 +94,45 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
     return out
 
 
+TOPK_MAX = 128
+
+
+def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspace=None, scratch=None):
+    """values, indices = top-k of the inference logits per row (what evaluate.py:158-159 computes as
+    xfc_forward(embed).topk(k)), without the dense [B, num_labels] matrix.  values bf16 [B, k] descending, indices int64
+    [B, k]; equal values are ordered by ascending label id."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dim() == 2 and x.shape[1] == FEATURES
+    assert 0 < k <= TOPK_MAX and k <= num_labels, "k must be between 1 and 128"
+    xb = x.to(torch.bfloat16).contiguous()      # exact for e4m3 input
+    arr, rows = _chunk_array(chunks)
+    nc = len(chunks)
+    if workspace is None:
+        workspace = alloc_workspace(nc, rows, x.device)
+    need = lib.xmc_topk_scratch_bytes(rows)
+    if scratch is None or scratch.numel() < need:
+        scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+    total = xb.shape[0]
+    vals = torch.empty(total, k, dtype=torch.bfloat16, device=x.device)
+    idx = torch.empty(total, k, dtype=torch.int32, device=x.device)
+    for lo in range(0, total, MAX_BATCH):
+        hi = min(lo + MAX_BATCH, total)
+        n = hi - lo
+        npad = (n + 15) // 16 * 16
+        xs = xb[lo:hi]
+        if npad != n:
+            xs = torch.cat([xs, torch.zeros(npad - n, FEATURES, dtype=xb.dtype, device=xb.device)])
+        tv = torch.empty(npad, k, dtype=torch.bfloat16, device=x.device)
+        ti = torch.empty(npad, k, dtype=torch.int32, device=x.device)
+        st = lib.xmc_fp8_forward_topk(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
+                                      int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
+                                      workspace.numel(), scratch.data_ptr(), scratch.numel(), _stream_ptr())
+        _lib.check(st, "xmc_fp8_forward_topk")
+        vals[lo:hi] = tv[:n]
+        idx[lo:hi] = ti[:n]
+    return vals, idx.to(torch.int64)
+
+
 WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}
 
 

@@ -101,6 +101,16 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
                                self._workspace)
 
     @torch.no_grad()
+    def xfc_forward_topk(self, embed, k):
+        '''
+        values, indices = xfc_forward(embed).topk(k) (what evaluate.py:158-159,235-236 compute) without the dense
+        [B, num_labels] logits: the top-k is merged chunk by chunk.  Not in the reference; k <= 128.
+        '''
+        assert embed.is_cuda and embed.dim() == 2
+        return ops.fp8_forward_topk(self._chunks(), embed, self.cfg.data.num_labels, k, self.scale_w, self.scale_x,
+                                    self._workspace)
+
+    @torch.no_grad()
     def _compute_loss(self, outlogit, rows, cols):
         '''
         BCE-with-logits summed over a dense logit block (reference :62-78; never reached in training because

@@ -74,6 +74,21 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one chunk and the running lists. */
+size_t xmc_topk_scratch_bytes(int rows_per_chunk);
+
+/* Inference with the top-k taken chunk by chunk: what the evaluation loop computes as
+ * xfc_forward(embed).topk(k) (evaluate.py:158-159,235-236 on chunked_fp8xmc_clf.py:45-60) without the dense
+ * [batch, num_labels] logits: the logits of one chunk at a time go to `scratch` and are merged into the k best per row.
+ *   out_val_bf16    device [batch, k] bf16, descending; equal values ordered by ascending label id
+ *   out_idx         device [batch, k] int32 label ids (< num_labels: the padding rows of the last chunk are dropped)
+ *   k               1..128, at most num_labels;  batch, x_bf16, scales, workspace: as xmc_fp8_forward
+ */
+int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                         int features, float scale_w, float scale_x, long long num_labels, int k, void* out_val_bf16,
+                         int32_t* out_idx, void* workspace, size_t workspace_bytes, void* scratch, size_t scratch_bytes,
+                         void* stream);
+
 /* Benchmarking aid (no counterpart in the reference): the next xmc_fp8_step call records these two HIP events
  * (hipEvent_t, created by the caller) immediately before and after its fused step kernel, on the call's stream,
  * then forgets them.  Pass nulls to cancel. */

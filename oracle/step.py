@@ -179,6 +179,22 @@ def fp8_forward(w_codes, x_any, num_labels, *, simulated=False, scale_w=1.0, sca
     return np.concatenate(outs, axis=1)[:, :num_labels]
 
 
+def topk_of_logits(logits_bf16, k):
+    """What evaluate.py:158-159,235-236 take from the dense logits of xfc_forward: the k largest per row, descending.
+    Ties are ordered by ascending label id (torch.topk leaves their order open).  NaN orders above every number, as in
+    torch.  Returns (values [B,k], indices [B,k] int64)."""
+    z = np.asarray(logits_bf16, dtype=np.float32)
+    key = np.where(np.isnan(z), np.float32(np.inf), z)
+    idx = np.arange(z.shape[1])
+    out_v = np.empty((z.shape[0], k), dtype=np.float32)
+    out_i = np.empty((z.shape[0], k), dtype=np.int64)
+    for b in range(z.shape[0]):
+        order = np.lexsort((idx, -key[b]))[:k]       # primary: value descending, secondary: label ascending
+        out_v[b] = z[b, order]
+        out_i[b] = order
+    return out_v, out_i
+
+
 def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rtn", return_parts=False,
               return_loss=False):
     """One step of the bf16 layer (chunked.py:85-131), weights bf16.

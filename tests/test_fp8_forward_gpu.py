@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 
 import helpers as H
+from elmo_amd import synth
 from oracle import codecs as C
 from oracle import step as O
 
@@ -38,3 +39,47 @@ def test_forward_scales(gpu):
     out = ops.fp8_forward(chunks, xd, 256, scale_w=2.0 ** -5, scale_x=0.25).float().cpu().numpy()
     ref = O.fp8_forward(case["chunks"], case["x"], 256, scale_w=2.0 ** -5, scale_x=0.25)
     H.assert_bf16_close(out, ref)
+
+
+@pytest.mark.parametrize("nc,rows,batch,num_labels,k", [
+    (1, 64, 16, 64, 5),             # a single tile, k small
+    (3, 2048, 48, 6000, 100),       # padding rows of the last chunk dropped
+    (2, 1024, 20, 2048, 128),       # batch padded to 32, largest k
+    (4, 4096, 128, 16000, 100),     # full batch
+    (2, 64, 16, 70, 70),            # k equal to the number of labels
+])
+def test_topk_forward(gpu, nc, rows, batch, num_labels, k):
+    """Chunk-wise top-k against the dense logits of the same library (bit-equal values, ids that point at them, the
+    documented order among ties) and against the oracle's top-k of the oracle's logits."""
+    import torch
+    from elmo_amd import ops
+    case = H.make_case(nc, rows, batch, 70 + nc, std=0.5)
+    chunks, x, _ = H.to_device_case(case, gpu)
+    dense = ops.fp8_forward(chunks, x, num_labels).float().cpu().numpy()
+    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k)
+    assert vals.shape == (batch, k) and idx.shape == (batch, k) and idx.dtype == torch.int64
+    v, i = vals.float().cpu().numpy(), idx.cpu().numpy()
+    want_v, want_i = O.topk_of_logits(dense, k)
+    assert np.array_equal(v, want_v)
+    assert np.array_equal(i, want_i)
+    assert i.min() >= 0 and i.max() < num_labels
+    # the oracle end to end: same values wherever its logits equal the library's
+    ref = O.fp8_forward(case["chunks"], case["x"], num_labels)
+    rv, ri = O.topk_of_logits(ref, k)
+    assert H.bf16_ulp_distance(v, rv).max() <= 1          # the logits themselves agree to one bf16 ulp
+    assert (i == ri).mean() > 0.8                         # a one-ulp difference can reorder near-ties
+
+
+def test_topk_with_repeated_values(gpu):
+    """Weights with few distinct values give logits with many exact ties across chunk boundaries."""
+    import torch
+    from elmo_amd import ops
+    rng = np.random.default_rng(3)
+    codes = rng.choice(np.array([0x30, 0xB0, 0x38, 0x00], dtype=np.uint8), size=(4096, 768))
+    codes[1000:3000] = codes[0:2000]                                   # identical rows in both chunks
+    case = dict(x=synth.make_x(16, 768, 5), chunks=[codes[:2048].copy(), codes[2048:].copy()], labels=np.zeros((0, 2), np.int32))
+    chunks, x, _ = H.to_device_case(case, gpu)
+    dense = ops.fp8_forward(chunks, x, 4096).float().cpu().numpy()
+    vals, idx = ops.fp8_forward_topk(chunks, x, 4096, 100)
+    want_v, want_i = O.topk_of_logits(dense, 100)
+    assert np.array_equal(vals.float().cpu().numpy(), want_v) and np.array_equal(idx.cpu().numpy(), want_i)

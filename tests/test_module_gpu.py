@@ -99,6 +99,12 @@ def test_evaluator_contract_and_checkpoint_roundtrip(gpu):
     H.assert_bf16_close(logits.float().cpu().numpy(), ref)
     ref_top = np.argsort(-ref, axis=1, kind="stable")[:, :5]
     assert np.mean(np.sort(ref_top, axis=1) == np.sort(idx.cpu().numpy(), axis=1)) > 0.97
+    # the same top-k without the dense logits: values equal, ids equal wherever the library routine's choice is unique
+    tv, ti = xfc.xfc_forward_topk(embed.to(xfc._dtype), 5)
+    assert torch.equal(tv, vals)
+    assert torch.equal(logits.gather(1, ti), vals) and ti.dtype == torch.int64
+    same = ti == idx
+    assert same.float().mean() > 0.9
     # runner.py:246 pickles xfc.xfc_weight with torch.save; :257 assigns it back
     buf = io.BytesIO()
     torch.save({"xfc_weight": xfc.xfc_weight, "model": xfc.state_dict()}, buf)

@@ -207,3 +207,24 @@ def test_loss_matches_the_library_routine_and_the_cited_op_sequence():
     want = torch.nn.functional.binary_cross_entropy_with_logits(
         torch.from_numpy(zall.astype(np.float64)), torch.from_numpy(y.astype(np.float64)), reduction="sum").item()
     assert abs(loss - want) <= 1e-9 * abs(want)
+
+
+def test_topk_matches_the_library_routine():
+    """topk_of_logits against torch.topk: identical values; identical indices where the values are distinct; and the
+    documented order among equal values."""
+    rng = np.random.default_rng(8)
+    z = C.bf16_round(rng.normal(0, 2.0, size=(6, 5000)).astype(np.float32))      # bf16 grid: many ties
+    v, i = O.topk_of_logits(z, 100)
+    tv, ti = torch.topk(torch.from_numpy(z), 100, dim=1)
+    assert np.array_equal(v, tv.numpy())
+    for b in range(z.shape[0]):
+        assert np.array_equal(z[b, i[b]], v[b]) and len(set(i[b].tolist())) == 100
+        same = v[b][1:] == v[b][:-1]
+        assert np.all(i[b][1:][same] > i[b][:-1][same])                        # ties: ascending label id
+        distinct = np.ones(100, bool); distinct[1:] &= ~same; distinct[:-1] &= ~same
+        below = (z[b] == v[b, -1]).sum() == (v[b] == v[b, -1]).sum()             # the last value may be cut among equals
+        keep = distinct & ((v[b] != v[b, -1]) | below)
+        assert np.array_equal(i[b][keep], ti[b].numpy()[keep])
+    tiny = np.array([[1.0, 3.0, 3.0, 2.0]], dtype=np.float32)
+    v, i = O.topk_of_logits(tiny, 3)
+    assert v.tolist() == [[3.0, 3.0, 2.0]] and i.tolist() == [[1, 2, 3]]
