@@ -369,13 +369,24 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       }
       tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
+    const int ugrid = 4 * ((tiles + TUP_TILES - 1) / TUP_TILES);
+#define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                          \
+  do {                                                                                                                           \
+    if (halves == 1)                                                                                                             \
+      tiled_update_kernel<WTYPE, RMODE, true><<<ugrid, 256, TUP_XBYTES, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr,   \
+                                                                                  seed, saturate, kahan, kahan_type, nh);       \
+    else                                                                                                                         \
+      tiled_update_kernel<WTYPE, RMODE, false><<<4 * tiles, 256, 0, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr, seed,\
+                                                                          saturate, kahan, kahan_type, nh);                     \
+  } while (0)
     if (weight_type == W_BF16) {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_BF16, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
-      else tiled_update_kernel<W_BF16, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_BF16, ROUND_RTN);
+      else XMC_LAUNCH_UPDATE(W_BF16, ROUND_SR_PHILOX);
     } else {
-      if (round_mode == XMC_ROUND_RTN) tiled_update_kernel<W_E4M3, ROUND_RTN><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
-      else tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX><<<4 * tiles, 256, 0, stream>>>(w, rows, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh);
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_RTN);
+      else XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_PHILOX);
     }
+#undef XMC_LAUNCH_UPDATE
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
   if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, 2 * num_tiles, loss_out);

@@ -448,12 +448,32 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
   }
 }
 
-template <int WT, int MODE>
-__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, const unsigned short* glb, size_t g_half_stride,
+constexpr int TUP_TILES = 4;                       // tiles of 64 label rows per workgroup when the operand is staged in LDS
+constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of one feature quarter and batch half: 48 KiB
+
+template <int WT, int MODE, bool XLDS>
+__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
                                                            int halves, const unsigned short* xT, float lr, unsigned seed,
                                                            int saturate, void* kahan, int kahan_type, int num_head) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
+  __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fb = blockIdx.x & 3, tile = blockIdx.x >> 2;
+  const int fb = blockIdx.x & 3, group = blockIdx.x >> 2;
+  // XLDS (one batch half): the X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and
+  // serves all tiles and wavefronts of the workgroup; from global memory every MFMA fetches its operand through L1
+  // again.  With two halves the 96 KiB would leave one workgroup per compute unit, which costs more than it saves.
+  for (int hh = 0; XLDS && hh < halves; hh++) {
+    const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (TUP_XBYTES / 2));
+#pragma unroll
+    for (int s = 0; s < TUP_XBYTES / 16 / 256; s++)
+      *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + (tid + 256 * s) * 16) = src[tid + 256 * s];
+  }
+  __syncthreads();
+  constexpr int TPW = XLDS ? TUP_TILES : 1;
+#pragma unroll 1
+  for (int tt = 0; tt < TPW; tt++) {
+  const int tile = group * TPW + tt;
+  if (tile >= ntiles) break;
   const int row = tile * TL + 16 * wv + l16;
   const bool live = row < rows;
   const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
@@ -499,7 +519,9 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
         if (hh < halves) {
 #pragma unroll
           for (int ks = 0; ks < 4; ks++) {
-            const bf16x8 xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((fb * 12 + nn) * (BP / 32) + ks) * 64 + lane) * 8);
+            bf16x8 xa;
+            if (XLDS) xa = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES + ((nn * (BP / 32) + ks) * 64 + lane) * 16);
+            else xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((fb * 12 + nn) * (BP / 32) + ks) * 64 + lane) * 8);
             a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
           }
         }
@@ -521,6 +543,7 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, co
         if (kahan_type == 1) kdst[1] = intx4{(int)ko[4], (int)ko[5], (int)ko[6], (int)ko[7]};
       }
     }
+  }
   }
 }
 
