@@ -266,8 +266,14 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
     const int n = (int)(num_labels - base < rows_per_chunk ? num_labels - base : rows_per_chunk);   // padding rows are dropped
     fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
                                                        scale_w * scale_x, zbuf, rows_per_chunk, 0, n, batch);
-    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, rows_per_chunk, n, (int)base, k, have, run_val, run_idx);
-    have = have + n < k ? have + n : k;
+    int done = 0;
+    if (have < k && n > 8192) {   // a short prefix first: it leaves k entries whose smallest value bounds the rest
+      done = 4096;
+      topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, rows_per_chunk, done, (int)base, k, have, run_val, run_idx);
+      have = have + done < k ? have + done : k;
+    }
+    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf + done, rows_per_chunk, n - done, (int)base + done, k, have, run_val, run_idx);
+    have = have + (n - done) < k ? have + (n - done) : k;
   }
   topk_finish_kernel<<<(batch * k + 255) / 256, 256, 0, stream>>>(run_val, run_idx, batch, k, (unsigned short*)out_val_bf16, out_idx);
   return launch_status();

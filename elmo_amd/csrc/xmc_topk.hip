@@ -6,14 +6,23 @@
 // One workgroup per batch row.  Candidates = the k entries kept so far (from the chunks before, hence smaller label
 // ids) followed by the chunk's logits in label order.  Radix select on a 16-bit key that orders bf16 values (two passes
 // of 256 bins find the key T of the k-th largest), then everything above T is taken, entries equal to T are taken in
-// candidate order until k are full (ties go to the smaller label id), and the k entries are sorted by (value
-// descending, label ascending).  NaN orders above every number, as in torch.topk.
+// candidate order until k are full (ties go to the smaller label id: a second radix select, on the label, among the
+// chunk's entries equal to T), and the k entries are sorted by (value descending, label ascending).  NaN orders above every number, as in torch.topk.
+// Once k entries are kept, their smallest value is a lower bound of the final k-th value: one pass over the chunk
+// keeps only the logits at or above it, in LDS, and the selection passes run over that short list (the chunk is read
+// again by every pass only when more than TOPK_CAP logits reach the bound).  The first chunk is therefore fed in two
+// parts, a short prefix that fits the list and produces a bound, and the rest.
 #include "xmc_common.h"
 
 namespace xmc {
 
 constexpr int TOPK_MAX = 128;   // largest k
 constexpr int TOPK_NT = 256;
+template <int N> struct TopkBins { static constexpr int value = N; };
+typedef TopkBins<256> B256;
+typedef TopkBins<1024> B1024;
+constexpr int TOPK_CAP = 6144;  // chunk logits at or above the bound that one workgroup keeps in LDS
+constexpr int TOPK_SMALL = 512; // candidates (kept entries included) that are ranked directly
 
 // ascending key order == ascending value order
 __device__ __forceinline__ unsigned topk_key(unsigned short bits) {
@@ -23,124 +32,242 @@ __device__ __forceinline__ unsigned short topk_bits(unsigned key) {
   return (key & 0x8000u) ? (unsigned short)(key & 0x7FFFu) : (unsigned short)(~key & 0xFFFFu);
 }
 
-// z: this row's logits of the chunk at z + row*stride, n of them valid (n % 4 may be anything; stride % 4 == 0)
+// z: this row's logits of the chunk at z + row*stride, n of them valid (n < 2^18; stride % 4 == 0; z 8-byte aligned)
 // run_key/run_idx: [batch][TOPK_MAX] entries kept so far, `have` of them valid; updated in place, sorted
 __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned short* z, long long stride, int n, int label_base, int k,
                                                              int have, unsigned short* run_val, int* run_idx) {
-  __shared__ unsigned hist[256];
-  __shared__ unsigned scan[TOPK_NT];
-  __shared__ unsigned sel_key[TOPK_MAX];
-  __shared__ int sel_idx[TOPK_MAX];
-  __shared__ unsigned s_bin, s_above, s_count;
+  __shared__ unsigned hist[1024];
+  __shared__ __attribute__((aligned(16))) unsigned sel_key[TOPK_MAX];
+  __shared__ __attribute__((aligned(16))) int sel_idx[TOPK_MAX];
+  __shared__ __attribute__((aligned(16))) unsigned cand_key[TOPK_CAP];
+  __shared__ __attribute__((aligned(16))) int cand_idx[TOPK_CAP];   // index in the chunk (negative: an entry kept from earlier chunks)
+  __shared__ unsigned s_bin, s_above, s_count, s_ncand, wtot[TOPK_NT / 64];
   const int tid = threadIdx.x;
   const unsigned short* row = z + (size_t)blockIdx.x * stride;
   unsigned short* rv = run_val + (size_t)blockIdx.x * TOPK_MAX;
   int* ri = run_idx + (size_t)blockIdx.x * TOPK_MAX;
   const int total = n + have;
   const int kk = k < total ? k : total;
-  // thread t owns the chunk elements [lo, hi): contiguous, so that candidate order is label order
-  const int per = ((n + TOPK_NT - 1) / TOPK_NT + 3) & ~3;
-  const int lo = min(tid * per, n), hi = min(lo + per, n);
   const unsigned mykey = tid < have ? topk_key(rv[tid]) : 0u;   // this thread's entry of the running list
   const int myidx = tid < have ? ri[tid] : -1;
+  const unsigned floor_key = have >= k ? topk_key(rv[k - 1]) : 0u;   // the list is sorted: entry k-1 is its smallest
 
-  // visits every chunk element of this thread: f(key, index in chunk)
-  auto for_each = [&](auto f) {
-    int i = lo;
-    for (; i + 4 <= hi; i += 4) {
-      const uint2 v = *(const uint2*)(row + i);
-      f(topk_key((unsigned short)(v.x & 0xFFFFu)), i);
-      f(topk_key((unsigned short)(v.x >> 16)), i + 1);
-      f(topk_key((unsigned short)(v.y & 0xFFFFu)), i + 2);
-      f(topk_key((unsigned short)(v.y >> 16)), i + 3);
-    }
-    for (; i < hi; i++) f(topk_key(row[i]), i);
-  };
-  // finds, from the top, the bin in which the `want`-th candidate lies: s_bin, and s_above = candidates in higher bins
-  auto pick_bin = [&](unsigned want) {
-    __syncthreads();
-    if (tid == 0) {
-      unsigned above = 0;
-      int b = 255;
-      for (; b > 0; b--) {
-        if (above + hist[b] >= want) break;
-        above += hist[b];
+  // visits every chunk element once, the workgroup reading 2 KiB of consecutive logits at a time, sixteen such loads in
+  // flight (a compute unit runs one workgroup: nothing else hides the latency): f(key, index in chunk)
+  auto for_each_global = [&](auto f) {
+    constexpr int U = 16;
+    for (int base = 0; base < n; base += U * 4 * TOPK_NT) {
+      uint2 v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int i = base + u * 4 * TOPK_NT + 4 * tid;
+        v[u] = i + 4 <= n ? *(const uint2*)(row + i) : uint2{0u, 0u};
       }
-      s_bin = (unsigned)b;
-      s_above = above;
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const int i = base + u * 4 * TOPK_NT + 4 * tid;
+        if (i + 4 <= n) {
+          f(topk_key((unsigned short)(v[u].x & 0xFFFFu)), i);
+          f(topk_key((unsigned short)(v[u].x >> 16)), i + 1);
+          f(topk_key((unsigned short)(v[u].y & 0xFFFFu)), i + 2);
+          f(topk_key((unsigned short)(v[u].y >> 16)), i + 3);
+        } else {
+          for (int j = i; j < n; j++) f(topk_key(row[j]), j);
+        }
+      }
+    }
+  };
+  // one pass over the chunk keeps the logits at or above the bound (key, index) in LDS; the selection then runs over
+  // that list.  More than TOPK_CAP of them: every later pass reads the chunk again.
+  if (tid == 0) s_ncand = 0;
+  __syncthreads();
+  for_each_global([&](unsigned key, int i) {
+    const bool take = key >= floor_key;
+    const unsigned long long m = __ballot(take);   // lanes of this wavefront that are here and take
+    if (m != 0) {
+      const int lane = tid & 63, leader = __ffsll((long long)m) - 1;
+      unsigned base = 0;
+      if (lane == leader) base = atomicAdd(&s_ncand, (unsigned)__popcll(m));
+      base = __shfl(base, leader, 64);
+      const unsigned slot = base + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
+      if (take && slot < (unsigned)TOPK_CAP) {
+        cand_key[slot] = key;
+        cand_idx[slot] = i;
+      }
+    }
+  });
+  __syncthreads();
+  const bool listed = s_ncand <= (unsigned)TOPK_CAP;
+  const int ncand = listed ? (int)s_ncand : 0;
+  // rank of (key, idx) among m entries of (keys, idxs) in the order value descending, index ascending; m % 4 == 0
+  auto rank_among = [&](const unsigned* keys, const int* idxs, int m, unsigned key, int idx) {
+    int rank = 0;
+    for (int j = 0; j < m; j += 4) {
+      const uint4 kj = *(const uint4*)(keys + j);
+      const int4 ij = *(const int4*)(idxs + j);
+      rank += (kj.x > key || (kj.x == key && ij.x < idx)) ? 1 : 0;
+      rank += (kj.y > key || (kj.y == key && ij.y < idx)) ? 1 : 0;
+      rank += (kj.z > key || (kj.z == key && ij.z < idx)) ? 1 : 0;
+      rank += (kj.w > key || (kj.w == key && ij.w < idx)) ? 1 : 0;
+    }
+    return rank;
+  };
+  if (listed && ncand + have <= TOPK_SMALL) {
+    // few candidates (the usual case once a bound exists): the kept entries join the list, every entry finds its rank
+    // among all of them and the first kk are written in place.  Kept entries have the smaller label ids.
+    const int m = ncand + have, m4 = (m + 3) & ~3;
+    if (tid < have) {
+      cand_key[ncand + tid] = mykey;
+      cand_idx[ncand + tid] = myidx - label_base;
+    }
+    if (tid < m4 - m) {   // padding that ranks after everything
+      cand_key[m + tid] = 0u;
+      cand_idx[m + tid] = 0x7FFFFFFF;
+    }
+    __syncthreads();
+    for (int c = tid; c < m; c += TOPK_NT) {
+      const unsigned key = cand_key[c];
+      const int idx = cand_idx[c];
+      const int rank = rank_among(cand_key, cand_idx, m4, key, idx);
+      if (rank < kk) {
+        rv[rank] = topk_bits(key);
+        ri[rank] = label_base + idx;
+      }
+    }
+    if (tid >= kk && tid < TOPK_MAX) {
+      rv[tid] = 0xFF80;   // -inf
+      ri[tid] = -1;
+    }
+    return;
+  }
+  auto for_each = [&](auto f) {
+    if (listed) {
+      for (int j = tid; j < ncand; j += TOPK_NT) f(cand_key[j], cand_idx[j]);
+    } else {
+      for_each_global([&](unsigned key, int i) { if (key >= floor_key) f(key, i); });
+    }
+  };
+  auto clear_hist = [&]() {
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 4; q++) hist[tid + TOPK_NT * q] = 0;
+    __syncthreads();
+  };
+  // exclusive prefix sum of one value per thread over the workgroup (thread order), and the total
+  auto block_scan = [&](unsigned val, unsigned& total) {
+    const int lane = tid & 63, wave = tid >> 6;
+    unsigned x = val;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned y = __shfl_up(x, off, 64);
+      if (lane >= off) x += y;
+    }
+    __syncthreads();
+    if (lane == 63) wtot[wave] = x;
+    __syncthreads();
+    unsigned before = 0;
+    total = 0;
+#pragma unroll
+    for (int q = 0; q < TOPK_NT / 64; q++) {
+      if (q < wave) before += wtot[q];
+      total += wtot[q];
+    }
+    return before + x - val;
+  };
+  // the bin in which the `want`-th candidate lies, counting from the top (down) or from the bottom: s_bin; s_above =
+  // candidates in the bins before it.  Thread t looks at bins/256 consecutive bins in counting order.
+  auto pick_bin = [&](unsigned want, auto bins_c, bool from_top) {
+    __syncthreads();
+    constexpr int bins = decltype(bins_c)::value;
+    constexpr int per = bins / TOPK_NT;
+    unsigned local[4] = {0, 0, 0, 0}, sum = 0;
+#pragma unroll
+    for (int q = 0; q < per; q++) {
+      const int pos = tid * per + q;
+      local[q] = hist[from_top ? bins - 1 - pos : pos];
+      sum += local[q];
+    }
+    unsigned total;
+    unsigned before = block_scan(sum, total);
+    if (tid == 0 && (want == 0 || total < want)) {   // nothing asked for, or fewer candidates than asked: the last bin in order
+      s_bin = (unsigned)(want == 0 ? (from_top ? bins - 1 : 0) : (from_top ? 0 : bins - 1));
+      s_above = want == 0 ? 0u : total - hist[from_top ? 0 : bins - 1];
+    }
+    if (want > 0 && total >= want) {
+#pragma unroll
+      for (int q = 0; q < per; q++) {
+        if (before < want && want <= before + local[q]) {
+          const int pos = tid * per + q;
+          s_bin = (unsigned)(from_top ? bins - 1 - pos : pos);
+          s_above = before;
+        }
+        before += local[q];
+      }
     }
     __syncthreads();
   };
 
-  hist[tid] = 0;
-  __syncthreads();
+  clear_hist();
   for_each([&](unsigned key, int) { atomicAdd(&hist[key >> 8], 1u); });
   if (tid < have) atomicAdd(&hist[mykey >> 8], 1u);
-  pick_bin((unsigned)kk);
+  pick_bin((unsigned)kk, B256{}, true);
   const unsigned hi_bin = s_bin, above_hi = s_above;
-  __syncthreads();
-  hist[tid] = 0;
-  __syncthreads();
+  clear_hist();
   for_each([&](unsigned key, int) { if ((key >> 8) == hi_bin) atomicAdd(&hist[key & 255u], 1u); });
   if (tid < have && (mykey >> 8) == hi_bin) atomicAdd(&hist[mykey & 255u], 1u);
-  pick_bin((unsigned)kk - above_hi);
+  pick_bin((unsigned)kk - above_hi, B256{}, true);
   const unsigned T = (hi_bin << 8) | s_bin;
   const unsigned n_gt = above_hi + s_above;          // candidates above T: all taken
   const unsigned need_eq = (unsigned)kk - n_gt;      // candidates equal to T still to take, in candidate order
 
   // equal candidates of the running list come first
-  unsigned eq_run = 0;
   __syncthreads();
   if (tid == 0) s_count = 0;
-  scan[tid] = (tid < have && mykey == T) ? 1u : 0u;
-  __syncthreads();
-  if (tid == 0) {
-    unsigned c = 0;
-    for (int i = 0; i < have; i++) { unsigned f = scan[i]; scan[i] = c; c += f; }
-    s_above = c;   // reused: equal entries in the running list
-  }
-  __syncthreads();
-  eq_run = s_above;
+  unsigned eq_run;
+  const unsigned my_eq_rank = block_scan((tid < have && mykey == T) ? 1u : 0u, eq_run);   // the list is in candidate order
   const unsigned eq_from_run = eq_run < need_eq ? eq_run : need_eq;
   if (tid < have) {
-    if (mykey > T || (mykey == T && scan[tid] < need_eq)) {
+    if (mykey > T || (mykey == T && my_eq_rank < need_eq)) {
       const unsigned slot = atomicAdd(&s_count, 1u);
       sel_key[slot] = mykey;
       sel_idx[slot] = myidx;
     }
   }
-  __syncthreads();
-  // equal candidates of the chunk, in label order: exclusive scan of the per-thread counts
-  unsigned my_eq = 0;
-  for_each([&](unsigned key, int) { my_eq += key == T ? 1u : 0u; });
-  scan[tid] = my_eq;
-  __syncthreads();
-  if (tid == 0) {
-    unsigned c = 0;
-    for (int i = 0; i < TOPK_NT; i++) { unsigned f = scan[i]; scan[i] = c; c += f; }
+  // the chunk's candidates equal to T are taken up to the index limit that admits eq_chunk of them: a second radix
+  // select, on the index (high bits i >> 10, then the low 10 bits), over those candidates only
+  const unsigned eq_chunk = need_eq - eq_from_run;
+  int idx_limit = -1;   // equal candidates with index <= idx_limit are taken
+  if (eq_chunk > 0) {
+    clear_hist();
+    for_each([&](unsigned key, int i) { if (key == T) atomicAdd(&hist[i >> 10], 1u); });
+    pick_bin(eq_chunk, B256{}, false);
+    const unsigned hi_idx = s_bin, below_hi = s_above;
+    clear_hist();
+    for_each([&](unsigned key, int i) { if (key == T && (unsigned)(i >> 10) == hi_idx) atomicAdd(&hist[i & 1023], 1u); });
+    pick_bin(eq_chunk - below_hi, B1024{}, false);
+    idx_limit = (int)((hi_idx << 10) | s_bin);
   }
   __syncthreads();
-  unsigned eq_rank = scan[tid];
-  const unsigned eq_chunk = need_eq - eq_from_run;
   for_each([&](unsigned key, int i) {
-    bool take = key > T;
-    if (key == T) { take = eq_rank < eq_chunk; eq_rank++; }
-    if (take) {
+    if (key > T || (key == T && i <= idx_limit)) {
       const unsigned slot = atomicAdd(&s_count, 1u);
-      sel_key[slot] = key;
-      sel_idx[slot] = label_base + i;
+      if (slot < (unsigned)TOPK_MAX) {
+        sel_key[slot] = key;
+        sel_idx[slot] = label_base + i;
+      }
     }
   });
+  __syncthreads();
+  if (tid >= kk && tid < TOPK_MAX) {   // padding that ranks after everything
+    sel_key[tid] = 0u;
+    sel_idx[tid] = 0x7FFFFFFF;
+  }
   __syncthreads();
   // exactly kk entries: sort by (value descending, label ascending) through ranks
   if (tid < kk) {
     const unsigned key = sel_key[tid];
     const int idx = sel_idx[tid];
-    int rank = 0;
-    for (int j = 0; j < kk; j++) {
-      const unsigned kj = sel_key[j];
-      rank += (kj > key || (kj == key && sel_idx[j] < idx)) ? 1 : 0;
-    }
+    const int rank = rank_among(sel_key, sel_idx, (kk + 3) & ~3, key, idx);
     rv[rank] = topk_bits(key);
     ri[rank] = idx;
   }

@@ -83,3 +83,24 @@ def test_topk_with_repeated_values(gpu):
     vals, idx = ops.fp8_forward_topk(chunks, x, 4096, 100)
     want_v, want_i = O.topk_of_logits(dense, 100)
     assert np.array_equal(vals.float().cpu().numpy(), want_v) and np.array_equal(idx.cpu().numpy(), want_i)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("k", [100, 7])
+def test_topk_when_most_logits_tie(gpu, k):
+    """Nearly all rows of W are one and the same row: more logits reach the running bound than the selection keeps in
+    fast memory, and the k-th value is a tie of thousands that the label id has to break."""
+    from elmo_amd import ops
+    rng = np.random.default_rng(11)
+    rows, nc = 16384, 2
+    base = rng.choice(np.array([0x30, 0xB0, 0x38, 0x28], dtype=np.uint8), size=768)
+    codes = np.tile(base, (nc * rows, 1))
+    odd = rng.choice(nc * rows, size=60, replace=False)                # a few rows that differ, above or below the rest
+    codes[odd] = rng.choice(np.array([0x30, 0xB0, 0x38, 0x28], dtype=np.uint8), size=(60, 768))
+    case = dict(x=synth.make_x(24, 768, 6), chunks=[codes[:rows].copy(), codes[rows:].copy()], labels=np.zeros((0, 2), np.int32))
+    chunks, x, _ = H.to_device_case(case, gpu)
+    num_labels = nc * rows - 5
+    dense = ops.fp8_forward(chunks, x, num_labels).float().cpu().numpy()
+    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k)
+    want_v, want_i = O.topk_of_logits(dense, k)
+    assert np.array_equal(vals.float().cpu().numpy(), want_v) and np.array_equal(idx.cpu().numpy(), want_i)
