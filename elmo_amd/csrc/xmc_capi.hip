@@ -29,7 +29,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WT_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
     (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
@@ -221,12 +221,22 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
   unsigned char* ws = (unsigned char*)workspace;
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
-  const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
-  const int grid = tiles_per_chunk < 4 * di.cus ? tiles_per_chunk : 4 * di.cus;
-  for (int c = 0; c < num_chunks; c++)
-    fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
-                                                       scale_w * scale_x, (unsigned short*)out_bf16, out_stride,
-                                                       (long long)c * rows_per_chunk, num_labels, batch);
+  ForwardParams fp;
+  for (int c = 0; c < num_chunks; c++) fp.chunk[c] = (const unsigned char*)chunk_ptrs[c];
+  fp.rows_per_chunk = rows_per_chunk;
+  fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
+  const int last_chunk = (int)((num_labels - 1) / rows_per_chunk);
+  fp.tile_begin = 0;
+  fp.tile_end = last_chunk * fp.tiles_per_chunk + (int)((num_labels - (long long)last_chunk * rows_per_chunk + FT - 1) / FT);
+  fp.xq = ws + WS_XQ;
+  fp.zscale = scale_w * scale_x;
+  fp.out = (unsigned short*)out_bf16;
+  fp.out_stride = out_stride;
+  fp.col0 = 0;
+  fp.num_labels = num_labels;
+  fp.batch = batch;
+  const int grid = fp.tile_end < 2 * di.cus ? fp.tile_end : 2 * di.cus;   // two workgroups fit the LDS of a compute unit
+  fp8_forward_kernel<<<grid, NT, FWD_LDS, stream>>>(fp);
   return launch_status();
 }
 
@@ -257,15 +267,26 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   int* run_idx = (int*)(run_val + (size_t)BP * TOPK_MAX);
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
-  const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
-  const int grid = tiles_per_chunk < 4 * di.cus ? tiles_per_chunk : 4 * di.cus;
+  ForwardParams fp;
+  for (int c = 0; c < num_chunks; c++) fp.chunk[c] = (const unsigned char*)chunk_ptrs[c];
+  fp.rows_per_chunk = rows_per_chunk;
+  fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
+  fp.xq = ws + WS_XQ;
+  fp.zscale = scale_w * scale_x;
+  fp.out = zbuf;
+  fp.out_stride = rows_per_chunk;
+  fp.num_labels = num_labels;
+  fp.batch = batch;
   int have = 0;
   for (int c = 0; c < num_chunks; c++) {
     const long long base = (long long)c * rows_per_chunk;
     if (base >= num_labels) break;
     const int n = (int)(num_labels - base < rows_per_chunk ? num_labels - base : rows_per_chunk);   // padding rows are dropped
-    fp8_forward_kernel<<<grid, NT, WT_BYTES, stream>>>((const unsigned char*)chunk_ptrs[c], rows_per_chunk, ws + WS_XQ,
-                                                       scale_w * scale_x, zbuf, rows_per_chunk, 0, n, batch);
+    fp.tile_begin = c * fp.tiles_per_chunk;
+    fp.tile_end = fp.tile_begin + (n + FT - 1) / FT;
+    fp.col0 = base;
+    const int tiles = fp.tile_end - fp.tile_begin;
+    fp8_forward_kernel<<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, FWD_LDS, stream>>>(fp);
     int done = 0;
     if (have < k && n > 8192) {   // a short prefix first: it leaves k entries whose smallest value bounds the rest
       done = 4096;

@@ -17,7 +17,7 @@
 namespace xmc {
 
 constexpr int TOPK_MAX = 128;   // largest k
-constexpr int TOPK_NT = 256;
+constexpr int TOPK_NT = 1024;  // one workgroup per batch row: sixteen wavefronts keep enough loads in flight on its compute unit
 template <int N> struct TopkBins { static constexpr int value = N; };
 typedef TopkBins<256> B256;
 typedef TopkBins<1024> B1024;
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned shor
   const int myidx = tid < have ? ri[tid] : -1;
   const unsigned floor_key = have >= k ? topk_key(rv[k - 1]) : 0u;   // the list is sorted: entry k-1 is its smallest
 
-  // visits every chunk element once, the workgroup reading 2 KiB of consecutive logits at a time, sixteen such loads in
+  // visits every chunk element once, the workgroup reading 8 KiB of consecutive logits at a time, sixteen such loads in
   // flight (a compute unit runs one workgroup: nothing else hides the latency): f(key, index in chunk)
   auto for_each_global = [&](auto f) {
     constexpr int U = 16;
@@ -149,8 +149,7 @@ __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned shor
   };
   auto clear_hist = [&]() {
     __syncthreads();
-#pragma unroll
-    for (int q = 0; q < 4; q++) hist[tid + TOPK_NT * q] = 0;
+    for (int q = tid; q < 1024; q += TOPK_NT) hist[q] = 0;
     __syncthreads();
   };
   // exclusive prefix sum of one value per thread over the workgroup (thread order), and the total
@@ -175,16 +174,16 @@ __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned shor
     return before + x - val;
   };
   // the bin in which the `want`-th candidate lies, counting from the top (down) or from the bottom: s_bin; s_above =
-  // candidates in the bins before it.  Thread t looks at bins/256 consecutive bins in counting order.
+  // candidates in the bins before it.  Thread t looks at one bin (or bins / threads consecutive bins) in counting order.
   auto pick_bin = [&](unsigned want, auto bins_c, bool from_top) {
     __syncthreads();
     constexpr int bins = decltype(bins_c)::value;
-    constexpr int per = bins / TOPK_NT;
-    unsigned local[4] = {0, 0, 0, 0}, sum = 0;
+    constexpr int per = bins > TOPK_NT ? bins / TOPK_NT : 1;
+    unsigned local[per], sum = 0;
 #pragma unroll
     for (int q = 0; q < per; q++) {
       const int pos = tid * per + q;
-      local[q] = hist[from_top ? bins - 1 - pos : pos];
+      local[q] = pos < bins ? hist[from_top ? bins - 1 - pos : pos] : 0u;
       sum += local[q];
     }
     unsigned total;

@@ -74,7 +74,10 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
     if workspace is None:
         workspace = alloc_workspace(nc, rows, x.device)
     total = xb.shape[0]
-    out = torch.empty(total, num_labels, dtype=torch.bfloat16, device=x.device)
+    # like the reference, which returns outlogit[:, :num_labels] of the concatenated chunk outputs, the result is a
+    # view of a [B, num_chunks * rows] buffer: rows start on 32-byte boundaries, which the kernel's stores want
+    stride = nc * rows
+    out = torch.empty(total, stride, dtype=torch.bfloat16, device=x.device)
     for lo in range(0, total, MAX_BATCH):
         hi = min(lo + MAX_BATCH, total)
         n = hi - lo
@@ -82,16 +85,16 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
         xs = xb[lo:hi]
         if npad != n:
             xs = torch.cat([xs, torch.zeros(npad - n, FEATURES, dtype=xb.dtype, device=xb.device)])
-            tmp = torch.empty(npad, num_labels, dtype=torch.bfloat16, device=x.device)
+            tmp = torch.empty(npad, stride, dtype=torch.bfloat16, device=x.device)
         else:
             tmp = out[lo:hi]
         st = lib.xmc_fp8_forward(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
-                                 tmp.data_ptr(), num_labels, num_labels, workspace.data_ptr(), workspace.numel(),
+                                 tmp.data_ptr(), stride, num_labels, workspace.data_ptr(), workspace.numel(),
                                  _stream_ptr())
         _lib.check(st, "xmc_fp8_forward")
         if npad != n:
-            out[lo:hi] = tmp[:n]
-    return out
+            out[lo:hi, :num_labels] = tmp[:n, :num_labels]
+    return out[:, :num_labels]
 
 
 TOPK_MAX = 128

@@ -68,7 +68,8 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
 
 /* Inference logits (chunked_fp8xmc_clf.py:45-60): out[b, label] = bf16(scale * sum_k e4m3(X/scale_x)[b,k] * W[label,k])
  * for label < num_labels (the padding rows of the last chunk are dropped, :60).
- *   out_bf16        device [batch, out_stride] bf16, out_stride >= num_labels
+ *   out_bf16        device [batch, out_stride] bf16, out_stride >= num_labels; any alignment works, rows that start
+ *                   on 32-byte boundaries (out_stride % 16 == 0) are written fastest
  */
 int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
                     int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
