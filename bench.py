@@ -6,6 +6,9 @@ src/xmc_classifiers/chunked_fp8xmc_clf.py:81-123): X[128,768] bf16 resident in H
 resident in HBM, positives as COO int32.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2_fp8_670k] [--round sr_fast|sr_philox|rtn]
+
+--mode forward / forward_topk time the FP8 layer's inference instead (xfc_forward, chunked_fp8xmc_clf.py:45-60, and
+the top-100 that evaluate.py:158-159 takes of it); the default mode and the headline metric is the training step.
 """
 import argparse
 import ctypes
@@ -134,6 +137,70 @@ def bench_tiled(args, cfg):
     print(json.dumps(out))
 
 
+def bench_inference(args, cfg):
+    """Inference of the FP8 layer on the workload's weights: dense logits, or the top-100 per row merged chunk by
+    chunk.  Timed as whole calls with HIP events on the torch stream."""
+    import torch
+    from elmo_amd import ops, synth
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    nc = cfg.num_chunks
+    rows = padded_labels(cfg.num_labels, nc) // nc
+    gen = torch.Generator(device=dev).manual_seed(cfg.seed)
+    chunks = [(torch.randn(rows, cfg.dim, generator=gen, device=dev, dtype=torch.float32) * cfg.init_std).to(torch.float8_e4m3fn)
+              for _ in range(nc)]
+    batch = min(cfg.batch, ops.MAX_BATCH)
+    x = torch.from_numpy(synth.make_x(batch, cfg.dim, cfg.seed)).to(dev).to(torch.bfloat16)
+    ws = ops.alloc_workspace(nc, rows, dev)
+    k = 100
+    topk = args.mode == "forward_topk"
+    scratch = torch.empty(ops.topk_scratch_bytes(rows), dtype=torch.uint8, device=dev) if topk else None
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base_alloc = torch.cuda.memory_allocated()
+
+    def one_call():
+        if topk:
+            return ops.fp8_forward_topk(chunks, x, cfg.num_labels, k, workspace=ws, scratch=scratch)
+        return ops.fp8_forward(chunks, x, cfg.num_labels, workspace=ws)
+
+    for _ in range(args.warmup):
+        one_call()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        res = one_call()
+    e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    dev_ms = e0.elapsed_time(e1) / args.steps
+    extra = torch.cuda.max_memory_allocated() - base_alloc
+    del res
+    weight_bytes = float(cfg.num_labels) * cfg.dim
+    algo_bytes = weight_bytes + (batch * k * 6.0 if topk else 2.0 * batch * cfg.num_labels)
+    achieved = algo_bytes / (dev_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath) and not topk:
+        with open(tpath) as f:
+            traffic = json.load(f).get(f"fp8_forward_kernel:{cfg.name}:forward")
+    print(json.dumps({
+        "metric": "XMC classifier inference calls/sec, " + ("top-100 per row without the dense logits" if topk else "dense logits"),
+        "value": args.steps / elapsed, "unit": "calls/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 MFMA, fp32 accumulate, bf16 logits", "data": "synthetic",
+        "config": {"workload": cfg.name, "mode": args.mode, "labels": cfg.num_labels, "features": cfg.dim, "batch": batch,
+                   "chunks": nc, "rows_per_chunk": rows, "k": k if topk else None},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "fp8_forward_kernel" + (" + topk_chunk_kernel per chunk" if topk else ""),
+                     "kernel_ms": dev_ms, "algorithmic_bytes_per_launch": algo_bytes},
+        "memory_beyond_weights_mb": extra / 1e6,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,6 +208,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="cfg2_fp8_670k")
     ap.add_argument("--round", default="sr_fast", choices=["sr_fast", "sr_philox", "rtn"])
+    ap.add_argument("--mode", default="step", choices=["step", "forward", "forward_topk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only launch the library's plain copy kernel over MIB MiB five times (counter calibration) and exit")
@@ -158,6 +226,11 @@ def main():
     if cfg.batch > ops.MAX_BATCH_TILED:
         print(f"bench.py: config {cfg.name} is not runnable by this build (batch > {ops.MAX_BATCH_TILED})", file=sys.stderr)
         sys.exit(2)
+    if args.mode != "step":
+        if cfg.weights == "bf16":
+            print("bench.py: the inference modes time the FP8 layer", file=sys.stderr)
+            sys.exit(2)
+        return bench_inference(args, cfg)
     if cfg.weights == "bf16" or "simfp8" in cfg.name or cfg.batch > ops.MAX_BATCH:
         return bench_tiled(args, cfg)
     dev = torch.device("cuda:0")

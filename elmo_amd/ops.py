@@ -100,6 +100,13 @@ def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None)
 TOPK_MAX = 128
 
 
+def topk_scratch_bytes(rows_per_chunk):
+    """Size of the scratch buffer fp8_forward_topk works in (the logits of one chunk and the running lists)."""
+    n = _lib.load().xmc_topk_scratch_bytes(rows_per_chunk)
+    assert n > 0, "rows_per_chunk must be a positive multiple of 16"
+    return n
+
+
 def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspace=None, scratch=None):
     """values, indices = top-k of the inference logits per row (what evaluate.py:158-159 computes as
     xfc_forward(embed).topk(k)), without the dense [B, num_labels] matrix.  values bf16 [B, k] descending, indices int64
