@@ -95,7 +95,8 @@ def bench_tiled(args, cfg):
     grad = torch.empty(cfg.batch, cfg.dim, dtype=torch.bfloat16, device=dev)
     true_fp8 = not bf16 and "simfp8" not in cfg.name
     rng = np.random.default_rng(cfg.seed)
-    mode = "rtn" if args.round == "rtn" else "sr_philox"
+    # the reference's Philox recipe where it is the only stochastic mode (bf16 weights, simulated FP8)
+    mode = args.round if true_fp8 or args.round == "rtn" else "sr_philox"
 
     def one_step():
         ops.tiled_step(views, rows, wtype, x, labels, cfg.lr, seeds=rng.integers(0, 1_000_000, size=len(views)),

@@ -329,7 +329,8 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
   if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1 || nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
   if (weight_type != W_E4M3 && weight_type != W_BF16) return XMC_ERR_MODE;
-  if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX) return XMC_ERR_MODE;
+  if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX && round_mode != XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
+  if (round_mode == XMC_ROUND_SR_FAST && weight_type != W_E4M3) return XMC_ERR_MODE;   // the converter rounds to e4m3
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
   for (int c = 0; c < num_chunks; c++) {
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
@@ -401,16 +402,17 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   do {                                                                                                                           \
     if (halves == 1)                                                                                                             \
       tiled_update_kernel<WTYPE, RMODE, true><<<ugrid, 256, TUP_XBYTES, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr,   \
-                                                                                  seed, saturate, kahan, kahan_type, nh);       \
+                                                                                  seed, saturate, kahan, kahan_type, nh, label0); \
     else                                                                                                                         \
       tiled_update_kernel<WTYPE, RMODE, false><<<4 * tiles, 256, 0, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr, seed,\
-                                                                          saturate, kahan, kahan_type, nh);                     \
+                                                                          saturate, kahan, kahan_type, nh, label0);             \
   } while (0)
     if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_BF16, ROUND_RTN);
       else XMC_LAUNCH_UPDATE(W_BF16, ROUND_SR_PHILOX);
     } else {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_RTN);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_FAST);
       else XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_PHILOX);
     }
 #undef XMC_LAUNCH_UPDATE

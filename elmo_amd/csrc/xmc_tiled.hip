@@ -385,7 +385,7 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 // Four consecutive features of one row: old weights (bf16: two dwords, e4m3: one) and compensation terms in, new ones out.
 template <int WT, int MODE>
 __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const unsigned* kraw, bool head, int kahan_type, float lr,
-                                          unsigned off0, unsigned seed, int saturate, unsigned* wout, unsigned* kout) {
+                                          unsigned off0, unsigned fidx, unsigned seed, int saturate, unsigned* wout, unsigned* kout) {
   float wv4[4];
   if (WT == W_BF16) {
     wv4[0] = bf16_from_bits((unsigned short)(wraw[0] & 0xffffu)); wv4[1] = bf16_from_bits((unsigned short)(wraw[0] >> 16));
@@ -424,8 +424,18 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
       for (int e = 0; e < 4; e++) t[e] = clamp448(t[e]);
     }
     int packed = 0;   // without the clamp: torch's cast gives NaN above 464 and so does the converter
-    packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
-    packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
+    if (MODE == ROUND_SR_FAST) {
+      // the fused kernel's mode: the converter rounds stochastically on the e4m3 grid, one counter hash per four
+      // weights (fidx = global row * 192 + column / 4)
+      const unsigned hsh = fast_mix(fidx, seed);
+      packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[0], fast_word(hsh, 0), packed, 0);
+      packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[1], fast_word(hsh, 1), packed, 1);
+      packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[2], fast_word(hsh, 2), packed, 2);
+      packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[3], fast_word(hsh, 3), packed, 3);
+    } else {
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], packed, false);
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], packed, true);
+    }
     wout[0] = (unsigned)packed;
     if (head) {
       floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8(packed, true);
@@ -454,7 +464,7 @@ constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of 
 template <int WT, int MODE, bool XLDS>
 __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
                                                            int halves, const unsigned short* xT, float lr, unsigned seed,
-                                                           int saturate, void* kahan, int kahan_type, int num_head) {
+                                                           int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
@@ -529,8 +539,9 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, in
       // a[e] = A[label row][feature col0 + 4q + e]
       if (live) {
         const int wq = WT == W_BF16 ? 2 * q : q, kq = kahan_type == 1 ? 2 * q : q;
-        t_update4<WT, MODE>(a, wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q), seed,
-                            saturate, wo + wq, ko + kq);
+        t_update4<WT, MODE>(a, wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
+                            (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * q) >> 2), seed, saturate, wo + wq,
+                            ko + kq);
       }
     }
     if (live) {

@@ -149,11 +149,10 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
                                              round_mode=self.rounding, workspace=self._tiled_workspace)
         elif embed.shape[0] > ops.MAX_BATCH:
             # the fused kernel holds 128 batch rows; larger batches take the three-kernel path with the same arithmetic
-            # (logits from e4m3(X), saturating cast), which rounds with the reference's recipe or to nearest
+            # (logits from e4m3(X), saturating cast) and the same rounding modes and random words
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128"
-            mode = "rtn" if self.rounding == "rtn" else "sr_philox"
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
-                                             round_mode=mode, workspace=self._tiled_workspace, quantize_x=True,
+                                             round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
                                              saturate=True)
         else:
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,

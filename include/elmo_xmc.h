@@ -114,7 +114,8 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
- *   round_mode       XMC_ROUND_RTN or XMC_ROUND_SR_PHILOX; batch: 1..256, any value (processed in halves of 128 rows)
+ *   round_mode       XMC_ROUND_RTN, XMC_ROUND_SR_PHILOX, or (e4m3 weights only) XMC_ROUND_SR_FAST with the random words of
+ *                    xmc_fp8_step's mode of that name; batch: 1..256, any value (processed in halves of 128 rows)
  *   quantize_x       e4m3 weights: 0 = logits from the un-quantised X (simulated FP8), 1 = from e4m3(X) (true FP8, :101)
  *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
  *   kahan, kahan_type, num_head

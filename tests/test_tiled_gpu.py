@@ -331,6 +331,47 @@ def test_true_fp8_with_a_batch_of_256(gpu):
     H.assert_bf16_close(xfc.grad_input.float().cpu().numpy(), ref_gi)
 
 
+def test_true_fp8_fast_rounding_on_the_three_kernel_path(gpu):
+    """sr_fast with e4m3 weights: the same random words as the fused kernel (one hash per four weights of a global row),
+    so the result equals the oracle's exact stochastic rounding fed with those words, and - with at most 128 batch rows -
+    the fused kernel's own output except where the two paths' fp32 sums differ."""
+    from elmo_amd import ops
+    nc, rows = 2, 272
+    case = H.make_case(nc, rows, 160, 64, pos_mean=4.0)
+    seeds = [31337, 4242]
+
+    def rand_fn(c, offs):
+        r, k = offs // 768, offs % 768
+        return C.fast_sr_words(seeds[c], c * rows + r, k)
+
+    chunks, x, labels = H.to_device_case(case, gpu)
+    ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.05, seeds=seeds, round_mode="sr_fast", quantize_x=True, saturate=True)
+    ref, _, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="exact", rand_fn=rand_fn)
+    total = mism = 0
+    for a, b in zip(H.chunks_to_numpy(chunks), ref):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1
+        mism += int((d != 0).sum()); total += d.size
+    assert mism / total < 2e-3, (mism, total)
+    # bf16 weights have no such mode
+    w = torch_bf16_weights(gpu, 64)
+    with pytest.raises(AssertionError):
+        ops.tiled_step([w], 64, "bf16", x[:16], labels[:0], 0.05, seeds=[1], round_mode="sr_fast")
+
+    case = H.make_case(nc, rows, 64, 65)
+    c1, x1, l1 = H.to_device_case(case, gpu)
+    c2, _, _ = H.to_device_case(case, gpu)
+    ops.tiled_step(c1, rows, "e4m3", x1, l1, 0.05, seeds=seeds, round_mode="sr_fast", quantize_x=True, saturate=True)
+    ops.fp8_step(c2, x1, l1, 0.05, seeds=seeds, round_mode="sr_fast")
+    diff = sum(int((a != b).sum()) for a, b in zip(H.chunks_to_numpy(c1), H.chunks_to_numpy(c2)))
+    assert diff / (nc * rows * 768) < 2e-3
+
+
+def torch_bf16_weights(device, rows):
+    import torch
+    return torch.zeros(rows, 768, dtype=torch.bfloat16, device=device)
+
+
 def test_head_kahan_module(gpu):
     import types
     import torch
