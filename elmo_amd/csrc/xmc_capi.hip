@@ -35,6 +35,11 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
   }
   return cached[dev];
 }
@@ -397,16 +402,10 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       }
       tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
-    const int ugrid = 4 * ((tiles + TUP_TILES - 1) / TUP_TILES);
-#define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                          \
-  do {                                                                                                                           \
-    if (halves == 1)                                                                                                             \
-      tiled_update_kernel<WTYPE, RMODE, true><<<ugrid, 256, TUP_XBYTES, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr,   \
-                                                                                  seed, saturate, kahan, kahan_type, nh, label0); \
-    else                                                                                                                         \
-      tiled_update_kernel<WTYPE, RMODE, false><<<4 * tiles, 256, 0, stream>>>(w, rows, tiles, glb, g_half, halves, xT, lr, seed,\
-                                                                          saturate, kahan, kahan_type, nh, label0);             \
-  } while (0)
+    const int ugrid = 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
+#define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                        \
+  tiled_update_kernel<WTYPE, RMODE><<<ugrid, 256 * halves, (size_t)TUP_XBYTES * halves, stream>>>(                             \
+      w, rows, tiles, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh, label0)
     if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_BF16, ROUND_RTN);
       else XMC_LAUNCH_UPDATE(W_BF16, ROUND_SR_PHILOX);

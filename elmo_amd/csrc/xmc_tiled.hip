@@ -458,31 +458,31 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
   }
 }
 
-constexpr int TUP_TILES = 4;                       // tiles of 64 label rows per workgroup when the operand is staged in LDS
+constexpr int TUP_TILES = 4;                       // tiles of 64 label rows that each group of four wavefronts processes
 constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of one feature quarter and batch half: 48 KiB
 
-template <int WT, int MODE, bool XLDS>
-__global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
+// Launched with 256 threads per batch half and TUP_XBYTES of LDS per batch half: four wavefronts per tile, so that a
+// compute unit runs eight wavefronts with one batch half (two workgroups) as with two (one workgroup, two tiles at a time).
+template <int WT, int MODE>
+__global__ __launch_bounds__(256 * T_HALVES) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
                                                            int halves, const unsigned short* xT, float lr, unsigned seed,
                                                            int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
-  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int tid = threadIdx.x, wv = (tid >> 6) & 3, sub = tid >> 8, nsub = (int)blockDim.x >> 8;
+  const int lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, group = blockIdx.x >> 2;
-  // XLDS (one batch half): the X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and
-  // serves all tiles and wavefronts of the workgroup; from global memory every MFMA fetches its operand through L1
-  // again.  With two halves the 96 KiB would leave one workgroup per compute unit, which costs more than it saves.
-  for (int hh = 0; XLDS && hh < halves; hh++) {
+  // The X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and serves all tiles and
+  // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
+  for (int hh = 0; hh < halves; hh++) {
     const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (TUP_XBYTES / 2));
-#pragma unroll
-    for (int s = 0; s < TUP_XBYTES / 16 / 256; s++)
-      *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + (tid + 256 * s) * 16) = src[tid + 256 * s];
+    for (int s = tid; s < TUP_XBYTES / 16; s += (int)blockDim.x)
+      *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + s * 16) = src[s];
   }
   __syncthreads();
-  constexpr int TPW = XLDS ? TUP_TILES : 1;
 #pragma unroll 1
-  for (int tt = 0; tt < TPW; tt++) {
-  const int tile = group * TPW + tt;
+  for (int tt = 0; tt < TUP_TILES; tt++) {
+  const int tile = (group * TUP_TILES + tt) * nsub + sub;
   if (tile >= ntiles) break;
   const int row = tile * TL + 16 * wv + l16;
   const bool live = row < rows;
@@ -529,9 +529,7 @@ __global__ __launch_bounds__(256) void tiled_update_kernel(void* w, int rows, in
         if (hh < halves) {
 #pragma unroll
           for (int ks = 0; ks < 4; ks++) {
-            bf16x8 xa;
-            if (XLDS) xa = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES + ((nn * (BP / 32) + ks) * 64 + lane) * 16);
-            else xa = *(const bf16x8*)(xT + (size_t)hh * D * BP + ((size_t)((fb * 12 + nn) * (BP / 32) + ks) * 64 + lane) * 8);
+            const bf16x8 xa = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES + ((nn * (BP / 32) + ks) * 64 + lane) * 16);
             a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
           }
         }
