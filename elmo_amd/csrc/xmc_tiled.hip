@@ -64,8 +64,9 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
   }
   const int half = b >> 7, bh = b & 127;
   xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
-  // feature k = 192 fbk + 48 kgk + 4 nn + e sits in row 4 kgk + e of block 12 fbk + nn (see tiled_update_kernel)
-  const int fbk = k / 192, r = k - fbk * 192, kgk = r / 48, nn = (r - kgk * 48) >> 2, e = r & 3;
+  // feature k = 192 fbk + 64 c + 16 kgk + 4 q + e sits in row 4 kgk + e of block 12 fbk + 4 c + q: in the update kernel
+  // a lane then owns 16 consecutive features per step c, and the four lanes of a label row 64 consecutive bytes
+  const int fbk = k / 192, r = k - fbk * 192, kgk = (r >> 4) & 3, nn = 4 * (r >> 6) + ((r >> 2) & 3), e = r & 3;
   xT[(size_t)half * BP * D + ((size_t)((fbk * 12 + nn) * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
 }
 
@@ -374,8 +375,9 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 
 // ---- grad_W and the SGD update of one chunk, in place.  blockIdx = tile*4 + fb; wavefront w owns label rows 16w..16w+15
 //      of the tile and features 192fb.. (12 blocks of 16).  A^T[f][l] = sum_b X^T[f][b] G[l][b].  The rows of a feature
-//      block are permuted (row 4kg+e of block nn is feature 192fb + 48kg + 4nn + e, see tiled_prep_x_kernel) so that a
-//      lane ends up with 48 consecutive features of one label row and moves them 16 at a time.
+//      block are permuted (row 4kg+e of block nn = 4c+q is feature 192fb + 64c + 16kg + 4q + e, see tiled_prep_x_kernel)
+//      so that a lane ends up with 16 consecutive features of one label row per step c, and the four lanes of a row
+//      with 64 consecutive bytes.
 //        bf16 weights : a = bf16(A); t = w - lr*a; RTN: bf16(t);  SR: bits(t) + (philox(seed, l*768+f) & 0xFFFF), clear 16 bits
 //        e4m3 weights : t = w - lr*A;          RTN: e4m3(t); SR: add 20 bits, clear, same cast.  The cast is torch's (NaN above
 //                       464; simulated FP8, chunked_fp8xmc_clf.py:116) or saturating at +-448 (true FP8, fuse_kernel.py:35).
@@ -464,7 +466,7 @@ constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of 
 // Launched with 256 threads per batch half and TUP_XBYTES of LDS per batch half: four wavefronts per tile, so that a
 // compute unit runs eight wavefronts with one batch half (two workgroups) as with two (one workgroup, two tiles at a time).
 template <int WT, int MODE>
-__global__ __launch_bounds__(256 * T_HALVES) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
+__global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
                                                            int halves, const unsigned short* xT, float lr, unsigned seed,
                                                            int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
@@ -480,6 +482,27 @@ __global__ __launch_bounds__(256 * T_HALVES) void tiled_update_kernel(void* w, i
       *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + s * 16) = src[s];
   }
   __syncthreads();
+  // The G rows and the weights of the next tile are loaded before the products of the current one: a wavefront waits
+  // for memory once per launch, not four times per tile.
+  constexpr int WDW = WT == W_BF16 ? 8 : 4;   // dwords of 16 weights
+  bf16x8 gf_n[T_HALVES][4];
+  intx4 wr_n[3][WDW / 4];
+  auto load_tile = [&](int tile) {
+    const int row = tile * TL + 16 * wv + l16;
+    const bool live = tile < ntiles && row < rows;
+#pragma unroll
+    for (int hh = 0; hh < T_HALVES; hh++)
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++)
+        gf_n[hh][ks] = (hh < halves && tile < ntiles) ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 192 * fb + 64 * c + 16 * kg) * (WT == W_BF16 ? 2 : 1));
+#pragma unroll
+      for (int q = 0; q < WDW / 4; q++) wr_n[c][q] = live ? src[q] : intx4{0, 0, 0, 0};
+    }
+  };
+  load_tile(group * TUP_TILES * nsub + sub);
 #pragma unroll 1
   for (int tt = 0; tt < TUP_TILES; tt++) {
   const int tile = (group * TUP_TILES + tt) * nsub + sub;
@@ -489,35 +512,36 @@ __global__ __launch_bounds__(256 * T_HALVES) void tiled_update_kernel(void* w, i
   const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
   const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
   bf16x8 gf[T_HALVES][4];
+  intx4 wr_t[3][WDW / 4];
 #pragma unroll
   for (int hh = 0; hh < T_HALVES; hh++)
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++)
-      gf[hh][ks] = hh < halves ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
-  constexpr int WDW = WT == W_BF16 ? 8 : 4;   // dwords of 16 weights
-#pragma unroll 1
+    for (int ks = 0; ks < 4; ks++) gf[hh][ks] = gf_n[hh][ks];
+#pragma unroll
+  for (int c = 0; c < 3; c++)
+#pragma unroll
+    for (int q = 0; q < WDW / 4; q++) wr_t[c][q] = wr_n[c][q];
+  if (tt + 1 < TUP_TILES) load_tile(tile + nsub);
+#pragma unroll
   for (int c = 0; c < 3; c++) {               // 16 consecutive features of this lane's row at a time
-    const int col0 = 192 * fb + 48 * kg + 16 * c;
+    const int col0 = 192 * fb + 64 * c + 16 * kg;
     const size_t idx = (size_t)row * D + col0;
     unsigned wr[WDW], wo[WDW], kr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, ko[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int q = 0; q < WDW; q++) { wr[q] = 0; wo[q] = 0; }
-    if (live) {
-      const intx4* src = (const intx4*)((const unsigned char*)w + idx * (WT == W_BF16 ? 2 : 1));
+    for (int q = 0; q < WDW / 4; q++) {
+      const intx4 v = wr_t[c][q];
+      wr[4 * q] = (unsigned)v.x; wr[4 * q + 1] = (unsigned)v.y; wr[4 * q + 2] = (unsigned)v.z; wr[4 * q + 3] = (unsigned)v.w;
+    }
 #pragma unroll
-      for (int q = 0; q < WDW / 4; q++) {
-        const intx4 v = src[q];
-        wr[4 * q] = (unsigned)v.x; wr[4 * q + 1] = (unsigned)v.y; wr[4 * q + 2] = (unsigned)v.z; wr[4 * q + 3] = (unsigned)v.w;
-      }
-      if (head) {
-        const int kdw = kahan_type == 1 ? 8 : 4;
-        const intx4* ksrc = (const intx4*)((const unsigned char*)kahan + idx * (kahan_type == 1 ? 2 : 1));
-        const intx4 v0 = ksrc[0];
-        kr[0] = (unsigned)v0.x; kr[1] = (unsigned)v0.y; kr[2] = (unsigned)v0.z; kr[3] = (unsigned)v0.w;
-        if (kdw == 8) {
-          const intx4 v1 = ksrc[1];
-          kr[4] = (unsigned)v1.x; kr[5] = (unsigned)v1.y; kr[6] = (unsigned)v1.z; kr[7] = (unsigned)v1.w;
-        }
+    for (int q = 0; q < WDW; q++) wo[q] = 0;
+    if (live && head) {
+      const int kdw = kahan_type == 1 ? 8 : 4;
+      const intx4* ksrc = (const intx4*)((const unsigned char*)kahan + idx * (kahan_type == 1 ? 2 : 1));
+      const intx4 v0 = ksrc[0];
+      kr[0] = (unsigned)v0.x; kr[1] = (unsigned)v0.y; kr[2] = (unsigned)v0.z; kr[3] = (unsigned)v0.w;
+      if (kdw == 8) {
+        const intx4 v1 = ksrc[1];
+        kr[4] = (unsigned)v1.x; kr[5] = (unsigned)v1.y; kr[6] = (unsigned)v1.z; kr[7] = (unsigned)v1.w;
       }
     }
 #pragma unroll
