@@ -113,6 +113,10 @@ __device__ __forceinline__ void q_lds_load16_l2(const unsigned char* g, unsigned
   const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off sc1" : : "s"(ldsoff), "v"(g) : "memory", "m0");
 }
+__device__ __forceinline__ void q_lds_load16_l2_sbase(const unsigned char* base, unsigned off, unsigned ldsoff_) {
+  const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 sc1" : : "s"(ldsoff), "v"(off), "s"(base) : "memory", "m0");
+}
 // 4 bytes per lane at device scope into LDS at ldsoff + 4*lane
 __device__ __forceinline__ void q_lds_load4_l2(const void* g, unsigned ldsoff_) {
   const unsigned ldsoff = __builtin_amdgcn_readfirstlane(ldsoff_);
@@ -274,15 +278,21 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   // Per-lane source rows and byte offsets of the wave-wide pieces this wavefront loads (pieces v and v+8 of an image).
   // own-column image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 pieces of 1 KiB
   // own-rows image:   rows 16m..16m+15, 16 x 49 chunks of 16 bytes (48 data + 1 pad) = 13 pieces
-  int wrow[2], wcol_off[2], rrow[2], rcol_off[2];
+  // The byte offsets are kept per lane for full tiles (nearly all): issuing a piece then costs no vector instruction.
+  // A tile cut short by the end of its chunk recomputes them with the row clamped to the last valid one.
+  auto wcol_offset = [&](int s, int last_row) {
+    const int ch = (v + 8 * s) * 64 + lane, wr = ch / 13;
+    return (unsigned)(min(wr, last_row) * D + QCOLS * m + min(ch - wr * 13, 11) * 16);
+  };
+  auto rows_offset = [&](int s, int last_row) {
+    const int ch = (v + 8 * s) * 64 + lane, rr = ch / 49;
+    return (unsigned)(min(16 * m + min(rr, 15), last_row) * D + min(ch - rr * 49, 47) * 16);
+  };
+  unsigned woff_full[2], roff_full[2];
 #pragma unroll
   for (int s = 0; s < 2; s++) {
-    const int ch = (v + 8 * s) * 64 + lane;
-    wrow[s] = ch / 13;
-    wcol_off[s] = QCOLS * m + min(ch - wrow[s] * 13, 11) * 16;
-    const int rr = ch / 49;
-    rrow[s] = 16 * m + min(rr, 15);
-    rcol_off[s] = min(ch - rr * 49, 47) * 16;
+    woff_full[s] = wcol_offset(s, TL - 1);
+    roff_full[s] = rows_offset(s, TL - 1);
   }
   q_cdesc* cdesc = (q_cdesc*)p.desc;
   // tile index of position k in this quad's sequence; positions past the end fall back to tile 0, whose data is
@@ -290,19 +300,21 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   auto tile_at = [&](int k) { const int t = quad + nquads * k; return t < p.num_tiles ? t : 0; };
   auto wcol_piece = [&](int slot, const QTile& q, int s) {
     if (v + 8 * s >= 13) return;
-    const unsigned off = (unsigned)(min(wrow[s], q.rows_valid - 1) * D + wcol_off[s]);
-    q_lds_load16_sbase(q.base, off, (unsigned)(slot * QWC_BYTES + (v + 8 * s) * 1024));
+    if (q.rows_valid == TL) q_lds_load16_sbase(q.base, woff_full[s], (unsigned)(slot * QWC_BYTES + (v + 8 * s) * 1024));
+    else q_lds_load16_sbase(q.base, wcol_offset(s, q.rows_valid - 1), (unsigned)(slot * QWC_BYTES + (v + 8 * s) * 1024));
   };
   auto rows_piece = [&](int slot, const QTile& q, int s) {
     if (v + 8 * s >= 13) return;
-    const unsigned off = (unsigned)(min(rrow[s], q.rows_valid - 1) * D + rcol_off[s]);
-    q_lds_load16_sbase(q.base, off, (unsigned)(QLDS_R + slot * QROW_BYTES + (v + 8 * s) * 1024));
+    if (q.rows_valid == TL) q_lds_load16_sbase(q.base, roff_full[s], (unsigned)(QLDS_R + slot * QROW_BYTES + (v + 8 * s) * 1024));
+    else q_lds_load16_sbase(q.base, rows_offset(s, q.rows_valid - 1), (unsigned)(QLDS_R + slot * QROW_BYTES + (v + 8 * s) * 1024));
   };
   // the G tile of position i: 18 pieces of 1 KiB (pieces v, v+8, v+16)
-  const unsigned char* gsrc_lane = p.exch + (size_t)quad * QSLOTS * QG_BYTES + v * 1024 + lane * 16;
+  const unsigned char* gsrc_quad = p.exch + (size_t)quad * QSLOTS * QG_BYTES;   // wave-uniform; the lane part is an offset
+  const unsigned gsrc_lane = (unsigned)(v * 1024 + lane * 16);
   auto gather_piece = [&](int i, int slot, int s) {
     if (v + 8 * s >= QG_PIECES) return;
-    q_lds_load16_l2(gsrc_lane + (i & (QSLOTS - 1)) * QG_BYTES + s * 8192, (unsigned)(QLDS_G + slot * QG_BYTES + (v + 8 * s) * 1024));
+    q_lds_load16_l2_sbase(gsrc_quad + (i & (QSLOTS - 1)) * QG_BYTES + s * 8192, gsrc_lane,
+                          (unsigned)(QLDS_G + slot * QG_BYTES + (v + 8 * s) * 1024));
   };
   // snapshot of the four counters of iteration i (wavefront 0 only), read in the next iteration
   auto issue_snapshot = [&](int i) {
