@@ -82,6 +82,13 @@ int step_kernel_choice() {
 
 int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
 
+// xmc_fp8_forward_topk takes the chunks in groups: as many as give at most 2^17 labels (fewer, larger launches), one
+// chunk if it is larger than that by itself
+int topk_group(int rows_per_chunk) { const int g = (1 << 17) / rows_per_chunk; return g < 1 ? 1 : g; }
+size_t topk_zbuf_bytes(int rows_per_chunk) {
+  return ((size_t)BP * topk_group(rows_per_chunk) * rows_per_chunk * 2 + 255) / 256 * 256;
+}
+
 }  // namespace
 
 extern "C" {
@@ -247,8 +254,9 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
 
 size_t xmc_topk_scratch_bytes(int rows_per_chunk) {
   if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return 0;
-  // logits of one chunk [128][rows] bf16, then the running lists: values [128][128] bf16, label ids [128][128] int32
-  return ((size_t)BP * rows_per_chunk * 2 + 255) / 256 * 256 + (size_t)BP * TOPK_MAX * 2 + (size_t)BP * TOPK_MAX * 4;
+  // logits of one group of chunks [128][group * rows] bf16, then the running lists: values [128][128] bf16, label ids
+  // [128][128] int32
+  return topk_zbuf_bytes(rows_per_chunk) + (size_t)BP * TOPK_MAX * 2 + (size_t)BP * TOPK_MAX * 4;
 }
 
 int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
@@ -262,13 +270,14 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   if (scratch_bytes < xmc_topk_scratch_bytes(rows_per_chunk)) return XMC_ERR_WORKSPACE;
   if (num_labels <= 0 || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
   if (k <= 0 || k > TOPK_MAX || k > num_labels) return XMC_ERR_SHAPE;
+  if (rows_per_chunk > (1 << 18)) return XMC_ERR_RANGE;   // the selection kernel indexes a group of chunks with 18 bits
   if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;
   hipStream_t stream = (hipStream_t)stream_;
   unsigned char* ws = (unsigned char*)workspace;
   unsigned short* zbuf = (unsigned short*)scratch;
-  unsigned short* run_val = (unsigned short*)((unsigned char*)scratch + ((size_t)BP * rows_per_chunk * 2 + 255) / 256 * 256);
+  unsigned short* run_val = (unsigned short*)((unsigned char*)scratch + topk_zbuf_bytes(rows_per_chunk));
   int* run_idx = (int*)(run_val + (size_t)BP * TOPK_MAX);
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
@@ -278,27 +287,30 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
   fp.xq = ws + WS_XQ;
   fp.zscale = scale_w * scale_x;
+  const int group = topk_group(rows_per_chunk);
+  const long long group_rows = (long long)group * rows_per_chunk;
   fp.out = zbuf;
-  fp.out_stride = rows_per_chunk;
+  fp.out_stride = group_rows;
   fp.num_labels = num_labels;
   fp.batch = batch;
   int have = 0;
-  for (int c = 0; c < num_chunks; c++) {
+  for (int c = 0; c < num_chunks; c += group) {
     const long long base = (long long)c * rows_per_chunk;
     if (base >= num_labels) break;
-    const int n = (int)(num_labels - base < rows_per_chunk ? num_labels - base : rows_per_chunk);   // padding rows are dropped
+    const int n = (int)(num_labels - base < group_rows ? num_labels - base : group_rows);   // padding rows are dropped
+    const int full = n / rows_per_chunk, rest = n - full * rows_per_chunk;                   // whole chunks, rows of the last one
     fp.tile_begin = c * fp.tiles_per_chunk;
-    fp.tile_end = fp.tile_begin + (n + FT - 1) / FT;
+    fp.tile_end = fp.tile_begin + full * fp.tiles_per_chunk + (rest + FT - 1) / FT;
     fp.col0 = base;
     const int tiles = fp.tile_end - fp.tile_begin;
     fp8_forward_kernel<<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, FWD_LDS, stream>>>(fp);
     int done = 0;
     if (have < k && n > 8192) {   // a short prefix first: it leaves k entries whose smallest value bounds the rest
       done = 4096;
-      topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, rows_per_chunk, done, (int)base, k, have, run_val, run_idx);
+      topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, group_rows, done, (int)base, k, have, run_val, run_idx);
       have = have + done < k ? have + done : k;
     }
-    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf + done, rows_per_chunk, n - done, (int)base + done, k, have, run_val, run_idx);
+    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf + done, group_rows, n - done, (int)base + done, k, have, run_val, run_idx);
     have = have + (n - done) < k ? have + (n - done) : k;
   }
   topk_finish_kernel<<<(batch * k + 255) / 256, 256, 0, stream>>>(run_val, run_idx, batch, k, (unsigned short*)out_val_bf16, out_idx);

@@ -75,12 +75,13 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one chunk and the running lists. */
+/* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one group of chunks (up to 2^17 labels, or one
+ * chunk of up to 2^18 rows) and the running lists. */
 size_t xmc_topk_scratch_bytes(int rows_per_chunk);
 
 /* Inference with the top-k taken chunk by chunk: what the evaluation loop computes as
  * xfc_forward(embed).topk(k) (evaluate.py:158-159,235-236 on chunked_fp8xmc_clf.py:45-60) without the dense
- * [batch, num_labels] logits: the logits of one chunk at a time go to `scratch` and are merged into the k best per row.
+ * [batch, num_labels] logits: the logits of a few chunks at a time go to `scratch` and are merged into the k best per row.
  *   out_val_bf16    device [batch, k] bf16, descending; equal values ordered by ascending label id
  *   out_idx         device [batch, k] int32 label ids (< num_labels: the padding rows of the last chunk are dropped)
  *   k               1..128, at most num_labels;  batch, x_bf16, scales, workspace: as xmc_fp8_forward

@@ -1,7 +1,7 @@
 """The headline workload at its full size (670 091 labels, 11 chunks, batch 128), checked through properties that
 do not need the whole oracle: sampled label rows against the oracle (the update of a row depends only on that
-row, X and the positives), lr = 0 leaves every weight byte unchanged, grad_X against an fp32 library GEMM, and
-positives change exactly the rows they name."""
+row, X and the positives), lr = 0 leaves every weight byte unchanged, grad_X against an fp32 library GEMM,
+positives change exactly the rows they name, and the inference logits and their top-100 against library routines."""
 import numpy as np
 import pytest
 
@@ -27,6 +27,29 @@ def big(gpu):
     x = torch.from_numpy(x_np).to(gpu).to(torch.bfloat16)
     labels = torch.from_numpy(labels_np).to(gpu)
     return dict(cfg=cfg, nc=nc, rows=rows, chunks=chunks, x=x, labels=labels, x_np=x_np, labels_np=labels_np)
+
+
+def test_inference_topk_at_full_size(gpu, big):
+    """670 091 labels: the dense logits against an fp32 library GEMM on sampled columns, and the top-100 merged group by
+    group (two chunks per group here, the last group a single short chunk) against torch.topk of the dense logits:
+    identical values, ids that point at them, all below the label count."""
+    import torch
+    from elmo_amd import ops
+    cfg = big["cfg"]
+    dense = ops.fp8_forward(big["chunks"], big["x"], cfg.num_labels)
+    assert dense.shape == (128, cfg.num_labels)
+    xq = big["x"].to(torch.float8_e4m3fn).float()
+    for c in (0, 5, big["nc"] - 1):
+        n = min(big["rows"], cfg.num_labels - c * big["rows"])
+        ref = (xq @ big["chunks"][c].float().t())[:, :n]
+        got = dense[:, c * big["rows"]:c * big["rows"] + n].float()
+        assert (got - ref).abs().max().item() <= 2.0 ** -7 * ref.abs().max().item()     # one bf16 rounding of the logit
+    vals, idx = ops.fp8_forward_topk(big["chunks"], big["x"], cfg.num_labels, 100)
+    want = torch.topk(dense, 100, dim=1)
+    assert torch.equal(vals.view(torch.int16), want.values.contiguous().view(torch.int16))
+    assert int(idx.min()) >= 0 and int(idx.max()) < cfg.num_labels
+    assert torch.equal(torch.gather(dense, 1, idx).view(torch.int16), vals.view(torch.int16))
+    assert bool((idx.sort(dim=1).values[:, 1:] != idx.sort(dim=1).values[:, :-1]).all())   # no label twice
 
 
 def test_lr_zero_is_identity_and_gradx_matches_library_gemm(gpu, big):
