@@ -35,11 +35,15 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, T_HALVES * TUP_XBYTES);
+    const int upd_lds = T_HALVES * TUP_XBYTES;   // the two-half variants need more than the default 64 KiB
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_RTN, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_SR_PHILOX, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
   }
   return cached[dev];
 }
@@ -415,17 +419,32 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
     const int ugrid = 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
+#define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
+  tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, 256 * HV, (size_t)TUP_XBYTES * HV, stream>>>(                             \
+      w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0)
 #define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                        \
-  tiled_update_kernel<WTYPE, RMODE><<<ugrid, 256 * halves, (size_t)TUP_XBYTES * halves, stream>>>(                             \
-      w, rows, tiles, glb, g_half, halves, xT, lr, seed, saturate, kahan, kahan_type, nh, label0)
+  do {                                                                                                                         \
+    if (halves == 1) XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 1, false); else XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 2, false);            \
+  } while (0)
+#define XMC_LAUNCH_UPDATE_HEAD(RMODE)                                                                                          \
+  do {                                                                                                                         \
+    if (halves == 1) XMC_LAUNCH_UPDATE_K(W_E4M3, RMODE, 1, true); else XMC_LAUNCH_UPDATE_K(W_E4M3, RMODE, 2, true);            \
+  } while (0)
+    const bool with_head = kahan_type != 0 && nh > 0;   // only chunk 0 of the head-Kahan layer
     if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_BF16, ROUND_RTN);
       else XMC_LAUNCH_UPDATE(W_BF16, ROUND_SR_PHILOX);
+    } else if (with_head) {
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_HEAD(ROUND_RTN);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE_HEAD(ROUND_SR_FAST);
+      else XMC_LAUNCH_UPDATE_HEAD(ROUND_SR_PHILOX);
     } else {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_RTN);
       else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_FAST);
       else XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_PHILOX);
     }
+#undef XMC_LAUNCH_UPDATE_HEAD
+#undef XMC_LAUNCH_UPDATE_K
 #undef XMC_LAUNCH_UPDATE
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);

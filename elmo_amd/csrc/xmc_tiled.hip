@@ -464,11 +464,14 @@ constexpr int TUP_TILES = 4;                       // tiles of 64 label rows tha
 constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of one feature quarter and batch half: 48 KiB
 
 // Launched with 256 threads per batch half and TUP_XBYTES of LDS per batch half: four wavefronts per tile, so that a
-// compute unit runs eight wavefronts with one batch half (two workgroups) as with two (one workgroup, two tiles at a time).
-template <int WT, int MODE>
-__global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride,
-                                                           int halves, const unsigned short* xT, float lr, unsigned seed,
-                                                           int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
+// compute unit runs at least eight wavefronts with one batch half as with two (one workgroup, two tiles at a time).
+// HALVES (batch halves, 1 or 2) and KAHAN (a compensated head may be present) are template parameters: with run-time
+// branches around the products the compiler issued every LDS operand read right in front of its matrix instruction.
+template <int WT, int MODE, int HALVES, bool KAHAN>
+__global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_update_kernel(
+    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, unsigned seed,
+    int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
+  static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = (tid >> 6) & 3, sub = tid >> 8, nsub = (int)blockDim.x >> 8;
@@ -476,7 +479,8 @@ __global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w
   const int fb = blockIdx.x & 3, group = blockIdx.x >> 2;
   // The X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and serves all tiles and
   // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
-  for (int hh = 0; hh < halves; hh++) {
+#pragma unroll
+  for (int hh = 0; hh < HALVES; hh++) {
     const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (TUP_XBYTES / 2));
     for (int s = tid; s < TUP_XBYTES / 16; s += (int)blockDim.x)
       *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + s * 16) = src[s];
@@ -485,16 +489,16 @@ __global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w
   // The G rows and the weights of the next tile are loaded before the products of the current one: a wavefront waits
   // for memory once per launch, not four times per tile.
   constexpr int WDW = WT == W_BF16 ? 8 : 4;   // dwords of 16 weights
-  bf16x8 gf_n[T_HALVES][4];
+  bf16x8 gf_n[HALVES][4];
   intx4 wr_n[3][WDW / 4];
   auto load_tile = [&](int tile) {
     const int row = tile * TL + 16 * wv + l16;
     const bool live = tile < ntiles && row < rows;
 #pragma unroll
-    for (int hh = 0; hh < T_HALVES; hh++)
+    for (int hh = 0; hh < HALVES; hh++)
 #pragma unroll
       for (int ks = 0; ks < 4; ks++)
-        gf_n[hh][ks] = (hh < halves && tile < ntiles) ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
+        gf_n[hh][ks] = tile < ntiles ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 192 * fb + 64 * c + 16 * kg) * (WT == W_BF16 ? 2 : 1));
@@ -509,12 +513,12 @@ __global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w
   if (tile >= ntiles) break;
   const int row = tile * TL + 16 * wv + l16;
   const bool live = row < rows;
-  const bool head = WT == W_E4M3 && kahan_type != 0 && row < num_head;
+  const bool head = KAHAN && kahan_type != 0 && row < num_head;
   const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
-  bf16x8 gf[T_HALVES][4];
+  bf16x8 gf[HALVES][4];
   intx4 wr_t[3][WDW / 4];
 #pragma unroll
-  for (int hh = 0; hh < T_HALVES; hh++)
+  for (int hh = 0; hh < HALVES; hh++)
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) gf[hh][ks] = gf_n[hh][ks];
 #pragma unroll
@@ -544,24 +548,37 @@ __global__ __launch_bounds__(256 * T_HALVES, 3) void tiled_update_kernel(void* w
         kr[4] = (unsigned)v1.x; kr[5] = (unsigned)v1.y; kr[6] = (unsigned)v1.z; kr[7] = (unsigned)v1.w;
       }
     }
+    // the four 16-feature products of this step: sixteen operand reads in flight (a batch of four or two products),
+    // then their matrix instructions
+    floatx4 acc[4];
+    constexpr int QB = HALVES == 1 ? 4 : 2;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int nn = 4 * c + q;
-      floatx4 a = {0.f, 0.f, 0.f, 0.f};
+    for (int q0 = 0; q0 < 4; q0 += QB) {
+      bf16x8 xa[QB][HALVES][4];
 #pragma unroll
-      for (int hh = 0; hh < T_HALVES; hh++) {
-        if (hh < halves) {
+      for (int qq = 0; qq < QB; qq++)
 #pragma unroll
-          for (int ks = 0; ks < 4; ks++) {
-            const bf16x8 xa = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES + ((nn * (BP / 32) + ks) * 64 + lane) * 16);
-            a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, gf[hh][ks], a, 0, 0, 0);
-          }
-        }
+        for (int hh = 0; hh < HALVES; hh++)
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++)
+            xa[qq][hh][ks] = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES +
+                                                                                (((4 * c + q0 + qq) * (BP / 32) + ks) * 64 + lane) * 16);
+#pragma unroll
+      for (int qq = 0; qq < QB; qq++) {
+        floatx4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int hh = 0; hh < HALVES; hh++)
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[qq][hh][ks], gf[hh][ks], a, 0, 0, 0);
+        acc[q0 + qq] = a;
       }
-      // a[e] = A[label row][feature col0 + 4q + e]
-      if (live) {
+    }
+    // acc[q][e] = A[label row][feature col0 + 4q + e]
+    if (live) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
         const int wq = WT == W_BF16 ? 2 * q : q, kq = kahan_type == 1 ? 2 * q : q;
-        t_update4<WT, MODE>(a, wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
+        t_update4<WT, MODE>(acc[q], wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
                             (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * q) >> 2), seed, saturate, wo + wq,
                             ko + kq);
       }
