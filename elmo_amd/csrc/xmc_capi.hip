@@ -410,11 +410,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       if (weight_type == W_BF16) {
         if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        tiled_gradx_kernel<W_BF16><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
+        tiled_gradx_kernel<W_BF16><<<4 * splits, 256, TgxGeom<W_BF16>::LDS, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       } else {
         if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, 0, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
+        tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, TgxGeom<W_E4M3>::LDS, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       }
       tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }

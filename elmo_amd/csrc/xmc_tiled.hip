@@ -255,82 +255,93 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
 }
 
 // ---- grad_X partial of one label range: C[128 x 192] = G^T[128 x R] W[R x 192].  blockIdx = fb + 4*split; wavefront w
-//      owns features 192fb + 48w.. (3 blocks of 16) against all 8 batch blocks.  W goes through a wavefront-private LDS
-//      block and comes back transposed (ds_read_b64_tr_b16).
+//      owns features 192fb + 48w.. (3 blocks of 16) against all 8 batch blocks.  Steps of 32 label rows: the step's
+//      slice of W (32 rows x 192 features of this workgroup, whole 16-byte pieces of contiguous row segments) and its
+//      8 KiB of G^T in operand order go straight to LDS, two steps ahead, in a ring of three stages; a compute unit's
+//      memory path handles few cache lines per clock, and register loads in operand order touched four times as many.
+//      The W operand comes back transposed (ds_read_b64_tr_b8 + exact fp8->bf16, or ds_read_b64_tr_b16).
+template <int WT> struct TgxGeom {
+  static constexpr int ROWB = WT == W_BF16 ? 384 : 192;                  // bytes of this workgroup's features in one row
+  static constexpr int STRIDE = ROWB + 16;                                // LDS row stride
+  static constexpr int SLOTS = STRIDE / 16;                               // 16-byte slots per LDS row, the last one padding
+  static constexpr int WPIECES = (32 * SLOTS + 63) / 64;                  // wave-wide loads of the W slice (7 or 13)
+  static constexpr int PIECES = WPIECES + 8;                              // ... and of G^T
+  static constexpr int PER_WAVE = (PIECES + 3) / 4;                       // every wavefront issues this many per step (4 or 6)
+  static constexpr int WBYTES = WPIECES * 1024;
+  static constexpr int STAGE = WBYTES + 8192;
+  static constexpr int LDS = 3 * STAGE;
+};
+
 template <int WT>
 __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, const unsigned short* gbl,
                                                           floatx4* partial) {
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[4 * 32 * T_WS2];
-  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  typedef TgxGeom<WT> G;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
+  __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
+  const unsigned lds0 = (unsigned)(size_t)lds;
+  const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, split = blockIdx.x >> 2;
-  const int f0 = 192 * fb + 48 * wv;
-  __attribute__((address_space(3))) unsigned char* lw = (__attribute__((address_space(3))) unsigned char*)lds_raw + wv * 32 * T_WS2;
   floatx4 acc[8][3];
 #pragma unroll
   for (int mb = 0; mb < 8; mb++)
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lbeg = split * range, lend = min(lbeg + range, bound);   // bound: this chunk's rows rounded up to a tile
-  // The operands of step l0 + 32 are loaded into registers while step l0 computes.
-  constexpr int NW = WT == W_BF16 ? 3 : 2;   // 16-byte pieces of W per lane and step
-  intx4 wraw[NW], wnext[NW];
-  bf16x8 ga[8], gnext[8];
-  auto load_step = [&](int l0, intx4* wr, bf16x8* g) {
+  const int nsteps = lend > lbeg ? (lend - lbeg + 31) >> 5 : 0;
+  // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv+4, ...; indices past the last piece repeat it),
+  // so that "all but the newest PER_WAVE" means the step before has landed.  Steps past the end repeat the last one.
+  auto issue_step = [&](int st, int stage) {
+    const int l0 = lbeg + 32 * min(st, nsteps - 1);
 #pragma unroll
-    for (int s = 0; s < NW; s++) {
-      const int c = lane + 64 * s;
-      if (WT == W_BF16) {
-        const int row = c / 6, c16 = c - row * 6;
-        const int lr = min(l0 + row, rows - 1);
-        wr[s] = *(const intx4*)((const unsigned short*)w + (size_t)lr * D + f0 + 8 * c16);
+    for (int j = 0; j < G::PER_WAVE; j++) {
+      const int piece = min(wv + 4 * j, G::PIECES - 1);
+      if (piece < G::WPIECES) {
+        const int ch = min(piece * 64 + lane, 32 * G::SLOTS - 1), row = ch / G::SLOTS, c16 = min(ch - row * G::SLOTS, G::SLOTS - 2);
+        const int lr = min(l0 + row, rows - 1);   // rows past the end re-read a valid one (their G is zero)
+        t_lds_load16((const unsigned char*)w + ((size_t)lr * D + 192 * fb) * (WT == W_BF16 ? 2 : 1) + 16 * c16,
+                     lds0 + (unsigned)(stage * G::STAGE + piece * 1024));
       } else {
-        const int cc = min(c, 95), row = cc / 3, c16 = cc - row * 3;
-        const int lr = min(l0 + row, rows - 1);
-        wr[s] = *(const intx4*)((const unsigned char*)w + (size_t)lr * D + f0 + 16 * c16);
+        const int gp = piece - G::WPIECES;
+        t_lds_load16((const unsigned char*)(gbl + ((size_t)((l0 >> 5) * 8 + gp) * 64 + lane) * 8),
+                     lds0 + (unsigned)(stage * G::STAGE + G::WBYTES + gp * 1024));
       }
     }
-#pragma unroll
-    for (int mb = 0; mb < 8; mb++) g[mb] = *(const bf16x8*)(gbl + ((size_t)((l0 >> 5) * 8 + mb) * 64 + lane) * 8);
   };
-  if (lbeg < lend) load_step(lbeg, wnext, gnext);
-  for (int l0 = lbeg; l0 < lend; l0 += 32) {
+  if (nsteps > 0) {
+    issue_step(0, 0);
+    issue_step(1, 1);
+  }
+  int stage = 0;
+  for (int st = 0; st < nsteps; st++) {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(G::PER_WAVE) : "memory");
+    __syncthreads();   // step st has landed for every wavefront; the stage of step st-1 is free
+    issue_step(st + 2, stage == 0 ? 2 : stage - 1);
+    const __attribute__((address_space(3))) unsigned char* wt = lds + stage * G::STAGE;
+    const __attribute__((address_space(3))) unsigned char* gt = wt + G::WBYTES;
+    bf16x8 ga[8];
 #pragma unroll
-    for (int s = 0; s < NW; s++) wraw[s] = wnext[s];
-#pragma unroll
-    for (int mb = 0; mb < 8; mb++) ga[mb] = gnext[mb];
-    if (l0 + 32 < lend) load_step(l0 + 32, wnext, gnext);
-    // W[l0..l0+31][f0..f0+47] -> LDS as bf16, row stride T_WS2 (the wavefront's own block: no barrier needed)
-    if (WT == W_BF16) {
-#pragma unroll
-      for (int s = 0; s < 3; s++) {
-        const int c = lane + 64 * s, row = c / 6, c16 = c - row * 6;
-        *(__attribute__((address_space(3))) intx4*)(lw + row * T_WS2 + c16 * 16) = wraw[s];
-      }
-    } else {
-#pragma unroll
-      for (int s = 0; s < 2; s++) {
-        const int c = lane + 64 * s;
-        if (c < 96) {
-          const int row = c / 3, c16 = c - row * 3;
-          const bf16x8 lo = t_fp8x8_to_bf16x8(intx2{wraw[s].x, wraw[s].y}), hi = t_fp8x8_to_bf16x8(intx2{wraw[s].z, wraw[s].w});
-          *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32) = lo;
-          *(__attribute__((address_space(3))) bf16x8*)(lw + row * T_WS2 + c16 * 32 + 16) = hi;
-        }
-      }
-    }
+    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + (mb * 64 + lane) * 16);
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
-      const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * T_WS2 + (16 * nn + 4 * (l16 & 3)) * 2);
-      tshortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(lw + off));
-      tshortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(lw + off + 4 * T_WS2));
-      wb[nn] = __builtin_bit_cast(bf16x8, tshortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+      if (WT == W_BF16) {
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * G::STRIDE + (48 * wv + 16 * nn + 4 * (l16 & 3)) * 2);
+        tshortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off));
+        tshortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off + 4 * G::STRIDE));
+        wb[nn] = __builtin_bit_cast(bf16x8, tshortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
+      } else {
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 1)) * G::STRIDE + 48 * wv + 16 * nn + (l16 & 1) * 8);
+        const intx2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(wt + off));
+        wb[nn] = t_fp8x8_to_bf16x8(raw);
+      }
     }
 #pragma unroll
     for (int mb = 0; mb < 8; mb++)
 #pragma unroll
       for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
+    stage = stage == 2 ? 0 : stage + 1;
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end still target LDS
   // acc[mb][nn][e] = C[batch 16mb + 4kg + e][feature f0 + 16nn + l16]
   floatx4* dst = partial + ((size_t)split * 4 + fb) * 24 * 256;
 #pragma unroll
