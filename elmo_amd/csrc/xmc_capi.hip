@@ -31,6 +31,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
     (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
+    (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
@@ -127,6 +128,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
   if (!grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
+  if (((uintptr_t)labels_coo & 7) != 0) return XMC_ERR_ALIGN;   // read as (row, label) pairs
   if (nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
   if (round_mode < XMC_ROUND_RTN || round_mode > XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
@@ -143,7 +145,8 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
   if (step_kernel_choice() == 1) {
-    (void)hipMemsetAsync(ws + WS_FLAGS, 0, 4096, stream);
+    // a fill kernel, not a memset node: the step may be recorded into a graph by the caller
+    tiled_zero_kernel<<<4, 256, 0, stream>>>((float*)(ws + WS_FLAGS), 1024);
     if (n_pad > 0)
       quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch,
                                                                             (unsigned*)(ws + WS_KEYS), nullptr);
@@ -206,7 +209,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
         labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
-    quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, 0, stream>>>(
+    quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, (size_t)(n_pad + 257) * 4, stream>>>(
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
         (unsigned short*)(ws + WS_XT));
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
@@ -238,7 +241,7 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
   ForwardParams fp;
-  for (int c = 0; c < num_chunks; c++) fp.chunk[c] = (const unsigned char*)chunk_ptrs[c];
+  for (int c = 0; c < MAX_CHUNKS; c++) fp.chunk[c] = c < num_chunks ? (const unsigned char*)chunk_ptrs[c] : nullptr;
   fp.rows_per_chunk = rows_per_chunk;
   fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
   const int last_chunk = (int)((num_labels - 1) / rows_per_chunk);
@@ -286,7 +289,7 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
   ForwardParams fp;
-  for (int c = 0; c < num_chunks; c++) fp.chunk[c] = (const unsigned char*)chunk_ptrs[c];
+  for (int c = 0; c < MAX_CHUNKS; c++) fp.chunk[c] = c < num_chunks ? (const unsigned char*)chunk_ptrs[c] : nullptr;
   fp.rows_per_chunk = rows_per_chunk;
   fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
   fp.xq = ws + WS_XQ;
@@ -357,7 +360,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
   }
-  if (!aligned16(x_bf16) || ((uintptr_t)workspace & 255) != 0) return XMC_ERR_ALIGN;
+  if (!aligned16(x_bf16) || ((uintptr_t)workspace & 255) != 0 || ((uintptr_t)labels_coo & 7) != 0) return XMC_ERR_ALIGN;
   if (workspace_bytes < xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk, batch)) return XMC_ERR_WORKSPACE;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;

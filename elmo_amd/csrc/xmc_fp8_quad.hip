@@ -170,29 +170,48 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
   if (blockIdx.x == 0 && flags)
     for (int i = tid; i < 1024; i += 256) flags[i] = 0;
   if (n_pad == 0) return;
-  for (int i = tid; i < n_pad; i += 256) {
-    unsigned key = 0xFFFFFFFFu;
-    if (i < nnz) {
-      int r = coo[2 * i], lab = coo[2 * i + 1];
-      if (r >= 0 && r < batch && lab >= 0 && lab < (1 << 24) - 1) key = ((unsigned)lab << 8) | (unsigned)r;
+  // eight (row, label) pairs per thread in flight at a time: the loads miss every cache
+  const int2* coo2 = (const int2*)coo;
+  for (int i0 = tid; i0 < n_pad; i0 += 8 * 256) {
+    int2 e[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int i = i0 + u * 256;
+      e[u] = i < nnz ? coo2[i] : int2{-1, -1};
     }
-    sk[i] = key;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int i = i0 + u * 256;
+      const int r = e[u].x, lab = e[u].y;
+      if (i < n_pad) sk[i] = (r >= 0 && r < batch && lab >= 0 && lab < (1 << 24) - 1) ? (((unsigned)lab << 8) | (unsigned)r) : 0xFFFFFFFFu;
+    }
   }
   __syncthreads();
   const int i0 = blockIdx.x * 64;
   const unsigned mine = sk[i0 + l];
   const int quarter = n_pad >> 2;
+  // keys in front of the workgroup's own 64 precede on <=, keys behind them on <, the own 64 by position; each part
+  // is a branch-free loop over groups of four so that several LDS reads are in flight
+  const int jb = w * quarter, je = (w + 1) * quarter;
+  const int e0 = min(je, max(jb, i0)), b2 = max(jb, min(je, i0 + 64));
+  const uint4* sk4 = (const uint4*)sk;
   int rank = 0;
-  for (int j = w * quarter; j < (w + 1) * quarter; j += 4) {   // groups of four never straddle the own range
-    const unsigned o0 = sk[j], o1 = sk[j + 1], o2 = sk[j + 2], o3 = sk[j + 3];
-    if (j < i0) {
-      rank += (o0 <= mine) + (o1 <= mine) + (o2 <= mine) + (o3 <= mine);
-    } else if (j >= i0 + 64) {
-      rank += (o0 < mine) + (o1 < mine) + (o2 < mine) + (o3 < mine);
-    } else {
-      const int me = i0 + l;
-      rank += (o0 < mine || (o0 == mine && j < me)) + (o1 < mine || (o1 == mine && j + 1 < me)) +
-              (o2 < mine || (o2 == mine && j + 2 < me)) + (o3 < mine || (o3 == mine && j + 3 < me));
+#pragma unroll 4
+  for (int j = jb >> 2; j < e0 >> 2; j++) {
+    const uint4 o = sk4[j];
+    rank += (o.x <= mine) + (o.y <= mine) + (o.z <= mine) + (o.w <= mine);
+  }
+#pragma unroll 4
+  for (int j = b2 >> 2; j < je >> 2; j++) {
+    const uint4 o = sk4[j];
+    rank += (o.x < mine) + (o.y < mine) + (o.z < mine) + (o.w < mine);
+  }
+  if (e0 < b2) {   // the part of the own 64 keys that lies in this wavefront's quarter
+    const int me = i0 + l;
+    for (int j = e0; j < b2; j += 4) {
+      const uint4 o = sk4[j >> 2];
+      rank += (o.x < mine || (o.x == mine && j < me)) + (o.y < mine || (o.y == mine && j + 1 < me)) +
+              (o.z < mine || (o.z == mine && j + 2 < me)) + (o.w < mine || (o.w == mine && j + 3 < me));
     }
   }
   unsigned* part = sk + n_pad;
@@ -215,22 +234,40 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
     prep_x_quad_thread(((int)blockIdx.x - desc_blocks) * 256 + (int)threadIdx.x, x, p.batch, inv_scale_x, xq, xt);
     return;
   }
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t > p.num_tiles) return;
-  auto lower = [&](int tt) {   // first key of tile tt (tt == num_tiles: first key past the last tile)
+  // the sorted keys go to LDS first (n_pad * 4 bytes, then 257 search results): a binary search in global memory
+  // is a chain of dependent cache misses
+  extern __shared__ unsigned dk[];
+  const int tid = threadIdx.x;
+  for (int i0 = tid; i0 < n_pad; i0 += 8 * 256) {
+    unsigned e[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) e[u] = i0 + u * 256 < n_pad ? p.keys[i0 + u * 256] : 0u;
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+      if (i0 + u * 256 < n_pad) dk[i0 + u * 256] = e[u];
+  }
+  __syncthreads();
+  int* found = (int*)(dk + n_pad);
+  const int t = blockIdx.x * 256 + tid;
+  auto lower = [&](int tt) {   // first key of tile tt (tt >= num_tiles: first key past the last tile)
+    if (tt > p.num_tiles) tt = p.num_tiles;
     const int c = tt / p.tiles_per_chunk, tj = tt - c * p.tiles_per_chunk;
     const unsigned long long bound = ((unsigned long long)c * p.rows_per_chunk + (unsigned long long)tj * TL) << 8;
     int lo = 0, hi = n_pad;
     while (lo < hi) {
       int mid = (lo + hi) >> 1;
-      if ((unsigned long long)p.keys[mid] < bound) lo = mid + 1; else hi = mid;
+      if ((unsigned long long)dk[mid] < bound) lo = mid + 1; else hi = mid;
     }
     return lo;
   };
   const int p0 = lower(t);
+  found[tid] = p0;
+  if (tid == 255) found[256] = lower(t + 1);
+  __syncthreads();
+  if (t > p.num_tiles) return;
   tile_ptr[t] = p0;
   if (t < p.num_tiles) {
-    const int p1 = lower(t + 1);
+    const int p1 = found[tid + 1];
     const int c = t / p.tiles_per_chunk;
     const int row0 = (t - c * p.tiles_per_chunk) * TL;
     const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);

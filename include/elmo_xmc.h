@@ -53,7 +53,8 @@ size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk);
  * SGD update (chunked_fp8xmc_clf.py:91-123).
  *   chunk_ptrs      host array of num_chunks device pointers, each [rows_per_chunk, 768] e4m3fn, updated in place
  *   x_bf16          device [batch, 768] bf16 (not modified); batch % 16 == 0, batch <= 128
- *   labels_coo      device [nnz, 2] int32 (row-in-batch, label id in the padded label space), any order, duplicates allowed
+ *   labels_coo      device [nnz, 2] int32 (row-in-batch, label id in the padded label space), any order, duplicates allowed;
+ *                   8-byte aligned (the pairs are read whole); entries outside the batch or the label space are ignored
  *   lr              learning rate (xmc_lr[0])
  *   seeds           host array of num_chunks seeds (one torch.randint(0, 1e6) per chunk in the reference, :113)
  *   round_mode      XMC_ROUND_*

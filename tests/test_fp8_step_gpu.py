@@ -111,3 +111,37 @@ def test_x_not_modified_and_deterministic(gpu):
     for a, b in zip(outs[0][0], outs[1][0]):
         assert torch.equal(a, b)
     assert torch.equal(outs[0][1], outs[1][1])      # fixed-order reduction: bitwise reproducible
+
+
+def test_step_replays_in_a_captured_graph(gpu):
+    """The step allocates nothing, never synchronises and clears its counters in a kernel, so a caller may record it
+    into a graph.  Three replays, with eager work and synchronisations between them, must give bit for bit what three
+    eager steps give (round-to-nearest, fixed-order grad_X)."""
+    import torch
+    from elmo_amd import ops
+    case = H.make_case(2, 4096, 128, 35)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    start = [c.view(torch.uint8).clone() for c in chunks]
+    ws = ops.alloc_workspace(len(chunks), chunks[0].shape[0], gpu)
+    gout = torch.empty(128, 768, dtype=torch.bfloat16, device=gpu)
+    eager = []
+    for _ in range(3):
+        ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws, grad_out=gout)
+        eager.append(([c.view(torch.uint8).clone() for c in chunks], gout.view(torch.int16).clone()))
+    for c, s in zip(chunks, start):
+        c.view(torch.uint8).copy_(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws, grad_out=gout)
+    for c, s in zip(chunks, start):      # the capture must not have run anything
+        assert torch.equal(c.view(torch.uint8), s)
+    for k in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ops.step_error_word(ws, len(chunks), chunks[0].shape[0]) == 0
+        for c, e in zip(chunks, eager[k][0]):
+            assert torch.equal(c.view(torch.uint8), e), f"weights differ after replay {k}"
+        assert torch.equal(gout.view(torch.int16), eager[k][1]), f"grad_input differs after replay {k}"
+        scratch = torch.randn(1 << 20, device=gpu).sum().item()      # unrelated eager work between the replays
+        assert scratch == scratch
