@@ -28,7 +28,7 @@ constexpr size_t TW_XT = TW_XB + (size_t)T_HALVES * BP * D * 2;    // X^T [halve
 constexpr size_t TW_KEYS = TW_XT + (size_t)T_HALVES * BP * D * 2;  // sorted positive keys
 constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [halves*128][768]
 constexpr size_t TW_PART = TW_GX + (size_t)T_HALVES * BP * D * 4;  // grad_X partials [T_SPLITS][128*768] fp32 (one half at a time)
-constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // per half: G [rows_pad][128] then G^T [128][rows_pad]; then tile_ptr
+constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr
 
 __device__ __forceinline__ bf16x8 t_fp8x8_to_bf16x8(intx2 raw) {
   bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
@@ -77,9 +77,11 @@ __global__ void tiled_zero_kernel(float* p, int n) {
 
 // ---- logits, sigmoid minus targets.  Persistent workgroups of 8 wavefronts; wavefront v keeps the X operand of batch
 //      rows 16v..16v+15 of this half in registers (96 of them) for the whole launch.  The label rows stream through LDS
-//      in sub-tiles of 32 rows (coalesced 16-byte loads into registers one sub-tile ahead, then LDS, two buffers, one
-//      barrier per sub-tile); every wavefront multiplies the sub-tile with its batch rows.  Writes G[l][b] row-major
-//      and G^T in the operand order of the grad_X kernel; rows beyond the chunk are written as zeros.
+//      in sub-tiles of 32 rows (direct-to-LDS loads two sub-tiles ahead, three buffers, one barrier per sub-tile);
+//      every wavefront multiplies the sub-tile with its batch rows.  Writes G twice, each in the operand order of its
+//      reader so that a wavefront's operand load there is 1 KiB of consecutive bytes: for the update kernel blocks of
+//      16 labels x 32 batch rows (lane = label + 16 * (batch row / 8), 8 batch rows per lane), for the grad_X kernel
+//      blocks of 16 batch rows x 32 labels; rows beyond the chunk are written as zeros.
 //      LOSS: also the sub-tile's share of the summed binary cross entropy of the bf16 logits z against the targets,
 //      sum over labels and batch rows of max(z, 0) - [positive] z + log(1 + exp(-|z|)), the quantity that
 //      _compute_loss of the reference is written to return (chunked.py:57-72), in fp32 and added per sub-tile for a
@@ -93,7 +95,8 @@ template <int WT> struct TlgGeom {
   static constexpr int BUF = PIECES * 1024;                              // bytes of one LDS buffer
   static constexpr int PER_WAVE = (PIECES + 7) / 8;                      // loads of wavefront 0 (7 or 4); the others issue at
   static constexpr int PER_WAVE_MIN = PIECES / 8;                        // least this many (6 or 3)
-  static constexpr int LDS = 3 * BUF + 64;                               // three buffers and eight partial sums of the loss
+  static constexpr int STAGE0 = 3 * BUF + 64;                            // 1 KiB per wavefront: its part of G, transposed
+  static constexpr int LDS = STAGE0 + 8 * 1024;                          // three buffers, eight partial sums of the loss, staging
 };
 
 // 16 bytes per lane from global memory straight into LDS at byte offset ldsoff + 16*lane (wave-uniform offset).  Inline
@@ -142,6 +145,7 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
   };
   const float nlog2e = -1.44269504088896340736f;
   const int gs = (int)gridDim.x;
+  __attribute__((address_space(3))) unsigned char* stg = lds + G::STAGE0 + v * 1024;
   issue_sub(blockIdx.x, 0);
   issue_sub(blockIdx.x + gs, 1);
   // the X operand of this wavefront's batch rows, behind the first two sub-tiles in the memory pipeline
@@ -153,8 +157,9 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
   for (int st = blockIdx.x; st < nsub; st += gs, it++) {
     // younger than the loads of this sub-tile: the loads of the next one and the stores of up to two steps
     if (it == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN) : "memory");
-    else if (it == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 10) : "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 20) : "memory");
+    // (three stores per wavefront and step: two of G^T, one of G)
+    else if (it == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 3) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 6) : "memory");
     // range of positives of the enclosing 64-row tile: asked for here, needed after the MFMAs
     const int p0 = ctile_ptr[st >> 1], p1 = ctile_ptr[(st >> 1) + 1];
     __syncthreads();
@@ -218,15 +223,24 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
       unsigned short sb[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[e]) : (unsigned short)0;
-      const int b = 16 * v + l16;
       uint2 o;
       o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
       o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
       // G^T in operand order for grad_X: block (label / 32, batch block) of 16 batch rows x 32 labels
       *(uint2*)(gbl + ((size_t)(st * 8 + v) * 64 + l16 + 16 * (2 * lb + (kg >> 1))) * 8 + 4 * (kg & 1)) = o;
+      // G for the update kernel: this wavefront's 32 labels x 16 batch rows, transposed through its own KiB of LDS
+      // (label-major, 32 bytes per label)
 #pragma unroll
-      for (int e = 0; e < 4; e++) glb[(size_t)(r0 + 4 * kg + e) * BP + b] = sb[e];
-
+      for (int e = 0; e < 4; e++)
+        *(__attribute__((address_space(3))) unsigned short*)(stg + (16 * lb + 4 * kg + e) * 32 + 2 * l16) = sb[e];
+    }
+    {
+      // ... and stored in the operand order of A = G X: block (16 labels, 32 batch rows) = 64 lanes x 8 batch rows,
+      // lane = label + 16 * (batch row / 8).  This wavefront's batch rows are half of K step v / 2: lanes 0..31 store
+      // the 512 contiguous bytes of the first label block, lanes 32..63 those of the second.
+      const int lbo = lane >> 5, half = (lane >> 4) & 1;
+      const uint4 gq = *(const __attribute__((address_space(3))) uint4*)(stg + (lane & 15) * 32 + 512 * lbo + 16 * half);
+      *(uint4*)(glb + ((size_t)((2 * st + lbo) * 4 + (v >> 1)) * 64 + (lane & 15) + 16 * (2 * (v & 1) + half)) * 8) = gq;
     }
     if (LOSS) {
       // lanes of a wavefront, then the eight wavefronts, in a fixed order; the halves of the batch run one after the other
@@ -509,7 +523,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
     for (int hh = 0; hh < HALVES; hh++)
 #pragma unroll
       for (int ks = 0; ks < 4; ks++)
-        gf_n[hh][ks] = tile < ntiles ? *(const bf16x8*)(glb + hh * g_half_stride + (size_t)row * BP + 32 * ks + 8 * kg) : bf16x8{};
+        gf_n[hh][ks] = tile < ntiles ? *(const bf16x8*)(glb + hh * g_half_stride + ((size_t)((tile * 4 + wv) * 4 + ks) * 64 + lane) * 8) : bf16x8{};
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 192 * fb + 64 * c + 16 * kg) * (WT == W_BF16 ? 2 : 1));

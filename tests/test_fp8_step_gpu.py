@@ -13,9 +13,12 @@ from oracle import step as O
 pytestmark = pytest.mark.gpu
 
 
-def run_rtn(case, device, lr=0.05, scale_w=1.0, scale_x=1.0):
+def run_rtn(case, device, lr=0.05, scale_w=1.0, scale_x=1.0, device_labels=None):
+    import torch
     from elmo_amd import ops
     chunks, x, labels = H.to_device_case(case, device)
+    if device_labels is not None:      # what the device is handed, when it differs from what the oracle is handed
+        labels = torch.from_numpy(np.ascontiguousarray(device_labels, dtype=np.int32)).to(device)
     ws = ops.alloc_workspace(len(chunks), chunks[0].shape[0], device)
     g, gf = ops.fp8_step(chunks, x, labels, lr, round_mode="rtn", scale_w=scale_w, scale_x=scale_x, workspace=ws,
                          want_f32=True)
@@ -83,6 +86,25 @@ def test_duplicate_and_dense_positives(gpu):
     extra = [(0, 0), (0, 0), (3, 0), (3, 5), (3, 5), (7, 63), (7, 64), (15, 127)] + [(b, 1) for b in range(16)]
     case = H.make_case(2, 64, 16, 31, extra_labels=extra)
     check_rtn(case, gpu)
+
+
+def test_many_positives_boundary_labels_and_ignored_entries(gpu):
+    """Close to the 16,384 pairs a step accepts (the sort and the descriptor search then use their largest LDS
+    footprint), with positives on the first and last label, on both sides of the chunk boundary and in every batch
+    row; pairs whose row or label lies outside the batch or the label space are ignored."""
+    nc, rows, batch = 2, 4096, 128
+    L = nc * rows
+    rng = np.random.default_rng(77)
+    flat = rng.choice(batch * L, size=16000, replace=False)
+    valid = np.stack([flat // L, flat % L], axis=1).astype(np.int32)
+    edge = np.array([[0, 0], [127, L - 1], [5, rows - 1], [5, rows], [64, rows - 1], [0, L - 1]], dtype=np.int32)
+    valid = np.concatenate([valid, edge], axis=0)
+    bogus = np.array([[-1, 3], [batch, 3], [255, 3], [1000, 3], [3, -5], [3, L], [3, (1 << 24) - 1], [3, 1 << 30]], dtype=np.int32)
+    mixed = np.concatenate([valid, bogus], axis=0)
+    mixed = mixed[rng.permutation(len(mixed))]
+    case = H.make_case(nc, rows, batch, 78)
+    case["labels"] = valid
+    check_rtn(case, gpu, device_labels=mixed)
 
 
 def test_no_positives(gpu):
