@@ -239,8 +239,8 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
       // lane = label + 16 * (batch row / 8).  This wavefront's batch rows are half of K step v / 2: lanes 0..31 store
       // the 512 contiguous bytes of the first label block, lanes 32..63 those of the second.
       const int lbo = lane >> 5, half = (lane >> 4) & 1;
-      const uint4 gq = *(const __attribute__((address_space(3))) uint4*)(stg + (lane & 15) * 32 + 512 * lbo + 16 * half);
-      *(uint4*)(glb + ((size_t)((2 * st + lbo) * 4 + (v >> 1)) * 64 + (lane & 15) + 16 * (2 * (v & 1) + half)) * 8) = gq;
+      const intx4 gq = *(const __attribute__((address_space(3))) intx4*)(stg + (lane & 15) * 32 + 512 * lbo + 16 * half);
+      *(intx4*)(glb + ((size_t)((2 * st + lbo) * 4 + (v >> 1)) * 64 + (lane & 15) + 16 * (2 * (v & 1) + half)) * 8) = gq;
     }
     if (LOSS) {
       // lanes of a wavefront, then the eight wavefronts, in a fixed order; the halves of the batch run one after the other
