@@ -221,6 +221,8 @@ def main():
 
     import numpy as np
     import torch
+    from elmo_amd import build as _build
+    _build.ensure_built()      # load what is built; compile only if there is nothing
     from elmo_amd import _lib, ops, synth
 
     cfg = synth.CONFIGS[args.config]

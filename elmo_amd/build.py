@@ -23,5 +23,10 @@ def build(verbose=False):
     return res.stderr if verbose else OUT
 
 
+def ensure_built():
+    """Builds the library only if none is there (tests, the smoke run and the benchmark load what is built)."""
+    return OUT if os.path.exists(OUT) else build()
+
+
 if __name__ == "__main__":
     print(build(verbose=True))

@@ -10,6 +10,8 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run on the GPU box only)")
+    from elmo_amd import build
+    build.ensure_built()      # the library in the tree is used as it is; it is compiled only if there is none
 
 
 @pytest.fixture(scope="session")
