@@ -61,6 +61,12 @@ size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk);
  *   scale_w/scale_x per-tensor scales: weight = scale_w * code, Xq = e4m3(X / scale_x); the reference uses 1, 1
  *   grad_x_bf16     device [batch, 768] bf16 out (self.grad_input, :122)
  *   grad_x_f32      device [batch, 768] fp32 out, or null
+ * Asynchronous on `stream`; allocates nothing and never synchronises.  The fused kernel is persistent: one workgroup
+ * per compute unit, and the four workgroups that share a tile stream wait for one another through counters in the
+ * workspace, so all of them must be running at the same time.  Give the step the whole device while it runs: a kernel
+ * of another stream that keeps compute units occupied for more than about ten milliseconds makes the waiting
+ * workgroups give up (every wait is bounded; nothing hangs) - the step's results are then invalid and the error word
+ * (xmc_step_error_word) is non-zero.  One step at a time per workspace.
  */
 int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
                  int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
@@ -147,7 +153,8 @@ int xmc_select_step_kernel(int which);
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
 
 /* Reads back the error word a step leaves in the workspace (non-zero: a workgroup gave up waiting for its
- * partner).  Synchronises the stream; meant for tests and debugging, not for the training loop. */
+ * partner, see xmc_fp8_step).  Synchronises the stream: meant for tests, debugging and an occasional check (say once
+ * per epoch, or where the training loop synchronises anyway), not for every step. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
 
 #ifdef __cplusplus
