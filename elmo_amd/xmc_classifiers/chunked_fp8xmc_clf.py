@@ -80,6 +80,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         # all scratch memory of the step comes from the torch allocator (so that max_memory_allocated sees it)
         self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
         self._tiled_workspace = None
+        self._fused_ran = False      # the error word in the workspace is defined once a fused step has run
         # batches of more than 128 rows (up to 256) also run on the three-kernel path, with the true-FP8 arithmetic
         self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
@@ -157,8 +158,17 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         else:
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
                                            scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
+            self._fused_ran = True
         self.iteration += 1
         return loss
+
+    def last_step_error(self):
+        """Error word of the last fused step (0 = fine; non-zero = a workgroup gave up waiting for its partners, e.g.
+        because another stream kept the device busy, and that step's results are invalid).  Synchronises the stream.
+        Not part of the reference's interface."""
+        if not self._fused_ran:
+            return 0
+        return ops.step_error_word(self._workspace, self.num_chunks, self.xfc_weight[0].shape[0])
 
     def filter_non_local_inds(self, rows, cols, start, end):
         mask = (cols >= start) & (cols < end)

@@ -152,9 +152,9 @@ int xmc_select_step_kernel(int which);
  * grid-stride kernel.  Memory-traffic counters are calibrated against this launch of known size. */
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
 
-/* Reads back the error word a step leaves in the workspace (non-zero: a workgroup gave up waiting for its
- * partner, see xmc_fp8_step).  Synchronises the stream: meant for tests, debugging and an occasional check (say once
- * per epoch, or where the training loop synchronises anyway), not for every step. */
+/* Reads back the error word the last step on this workspace left there (non-zero: a workgroup gave up waiting for its
+ * partner, see xmc_fp8_step; every step clears the word when it starts).  Synchronises the stream: meant for tests,
+ * debugging and a check where the training loop synchronises anyway, not for every step. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
 
 #ifdef __cplusplus

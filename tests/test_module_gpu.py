@@ -39,6 +39,7 @@ def test_construction_matches_reference_layout(gpu):
 def test_training_call_contract(gpu):
     import torch
     xfc = build(gpu, 1000, 2, rounding="rtn")
+    assert xfc.last_step_error() == 0                   # nothing has run yet
     enc = torch.nn.Linear(768, 768, bias=False).to(gpu).to(torch.bfloat16)
     torch.manual_seed(1)
     tokens = torch.randn(32, 768, device=gpu, dtype=torch.bfloat16)
@@ -51,6 +52,7 @@ def test_training_call_contract(gpu):
     grad_fn = out.grad_fn
     loss = xfc.xfc_forward_backward(out, labels, [0.05], skip_loss=True)
     assert loss == 0 and xfc.iteration == 1
+    assert xfc.last_step_error() == 0                   # no workgroup gave up waiting
     assert torch.equal(out.detach().view(torch.int16), out_copy.view(torch.int16)) and out.grad_fn is grad_fn
     g = xfc.grad_input
     assert g.shape == (32, 768) and g.dtype == out.dtype and g.is_cuda
