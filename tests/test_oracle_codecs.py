@@ -84,7 +84,7 @@ def test_philox_random123_known_answers(ctr, key, out):
 
 
 def test_tl_randint_recorded_words():
-    # words produced by Triton's tl.randint(seed=1024, offsets 0..3) (library routine, recorded in the survey)
+    # words produced by Triton's tl.randint(seed=1024, offsets 0..3) (library routine run through the interpreter, values recorded beforehand)
     assert list(C.tl_randint(1024, np.arange(4))) == [3876201247, 854061192, 798737492, 713463838]
 
 
@@ -127,7 +127,7 @@ def test_sr_exact_is_unbiased_everywhere_and_saturates():
     big = np.array([460.0, 1000.0, -1e9], dtype=np.float32)
     assert np.array_equal(C.e4m3_decode(C.sr_e4m3_exact(big, np.array([0xFFFFFFFF] * 3, dtype=np.uint64))),
                           np.array([448.0, 448.0, -448.0], dtype=np.float32))
-    # the reference recipe, by contrast, is biased below 2^-6: its final cast rounds to nearest (survey app. A4)
+    # the reference recipe, by contrast, is biased below 2^-6: its final cast rounds to nearest (fuse_kernel.py:29-36)
     t = np.full(1 << 20, 0.00097656 * 0.5, dtype=np.float32)
     ref = C.e4m3_decode(C.e4m3_encode(C.sr_add_mask(t, np.arange(1 << 20, dtype=np.uint64), 20))).astype(np.float64)
     assert abs(ref.mean() - float(t[0])) > 1e-4
