@@ -261,9 +261,9 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
 
 size_t xmc_topk_scratch_bytes(int rows_per_chunk) {
   if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return 0;
-  // logits of one group of chunks [128][group * rows] bf16, then the running lists: values [128][128] bf16, label ids
-  // [128][128] int32
-  return topk_zbuf_bytes(rows_per_chunk) + (size_t)BP * TOPK_MAX * 2 + (size_t)BP * TOPK_MAX * 4;
+  // logits of one group of chunks [128][group * rows] bf16, then the running lists, two per batch row: values
+  // [128][2][128] bf16, label ids [128][2][128] int32
+  return topk_zbuf_bytes(rows_per_chunk) + 2 * ((size_t)BP * TOPK_MAX * 2 + (size_t)BP * TOPK_MAX * 4);
 }
 
 int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
@@ -285,7 +285,7 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   unsigned char* ws = (unsigned char*)workspace;
   unsigned short* zbuf = (unsigned short*)scratch;
   unsigned short* run_val = (unsigned short*)((unsigned char*)scratch + topk_zbuf_bytes(rows_per_chunk));
-  int* run_idx = (int*)(run_val + (size_t)BP * TOPK_MAX);
+  int* run_idx = (int*)(run_val + (size_t)BP * 2 * TOPK_MAX);
   prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
                                                               (unsigned short*)(ws + WS_XT));
   ForwardParams fp;
@@ -300,7 +300,17 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   fp.out_stride = group_rows;
   fp.num_labels = num_labels;
   fp.batch = batch;
-  int have = 0;
+  // Every batch row keeps two lists.  Large groups are split between two workgroups per row (one list each), so that
+  // 128 rows occupy all compute units; small ones go to list 0.  A list without k entries yet is first given a short
+  // piece (4,096 logits, which fit the workgroup's candidate store): that leaves k entries whose smallest value bounds
+  // the rest.
+  int have[2] = {0, 0};
+  auto select = [&](const unsigned short* zp, int n, int base, int parts) {
+    topk_chunk_kernel<<<batch * parts, TOPK_NT, 0, stream>>>(zp, group_rows, n, base, k, parts, have[0], have[1], run_val, run_idx);
+    const int n0 = parts == 2 ? topk_split(n) : n;
+    have[0] = have[0] + n0 < k ? have[0] + n0 : k;
+    have[1] = have[1] + (n - n0) < k ? have[1] + (n - n0) : k;
+  };
   for (int c = 0; c < num_chunks; c += group) {
     const long long base = (long long)c * rows_per_chunk;
     if (base >= num_labels) break;
@@ -312,15 +322,21 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
     const int tiles = fp.tile_end - fp.tile_begin;
     fp8_forward_kernel<<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, FWD_LDS, stream>>>(fp);
     int done = 0;
-    if (have < k && n > 8192) {   // a short prefix first: it leaves k entries whose smallest value bounds the rest
-      done = 4096;
-      topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf, group_rows, done, (int)base, k, have, run_val, run_idx);
-      have = have + done < k ? have + done : k;
+    if (n > 32768) {          // two workgroups per row
+      if (have[0] < k || have[1] < k) {
+        done = 8192;
+        select(zbuf, done, (int)base, 2);
+      }
+      select(zbuf + done, n - done, (int)base + done, 2);
+    } else {
+      if (have[0] < k && n > 8192) {
+        done = 4096;
+        select(zbuf, done, (int)base, 1);
+      }
+      select(zbuf + done, n - done, (int)base + done, 1);
     }
-    topk_chunk_kernel<<<batch, TOPK_NT, 0, stream>>>(zbuf + done, group_rows, n - done, (int)base + done, k, have, run_val, run_idx);
-    have = have + (n - done) < k ? have + (n - done) : k;
   }
-  topk_finish_kernel<<<(batch * k + 255) / 256, 256, 0, stream>>>(run_val, run_idx, batch, k, (unsigned short*)out_val_bf16, out_idx);
+  topk_finish_kernel<<<batch, 2 * TOPK_MAX, 0, stream>>>(run_val, run_idx, k, have[0], have[1], (unsigned short*)out_val_bf16, out_idx);
   return launch_status();
 }
 

@@ -32,10 +32,15 @@ __device__ __forceinline__ unsigned short topk_bits(unsigned key) {
   return (key & 0x8000u) ? (unsigned short)(key & 0x7FFFu) : (unsigned short)(~key & 0xFFFFu);
 }
 
-// z: this row's logits of the chunk at z + row*stride, n of them valid (n < 2^18; stride % 4 == 0; z 8-byte aligned)
-// run_key/run_idx: [batch][TOPK_MAX] entries kept so far, `have` of them valid; updated in place, sorted
-__global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned short* z, long long stride, int n, int label_base, int k,
-                                                             int have, unsigned short* run_val, int* run_idx) {
+// z: a row's logits of the chunk at z + row*stride, n_all of them valid (n_all < 2^18; stride % 4 == 0; z 8-byte aligned)
+// run_val/run_idx: [batch][2][TOPK_MAX] entries kept so far: every batch row has two lists, which topk_finish_kernel
+// merges.  parts = 1: one workgroup per row adds all n_all logits to list 0 (have0 entries valid).  parts = 2: two
+// workgroups per row, so that 128 rows fill 256 compute units; workgroup 2 row + p takes the first topk_split(n_all)
+// logits (p = 0) or the rest (p = 1) and updates list p (have0 / have1 entries valid).  Lists are updated in place and
+// stay sorted; within a list the entries kept from earlier launches have the smaller label ids.
+__host__ __device__ __forceinline__ int topk_split(int n_all) { return ((n_all >> 1) + 3) & ~3; }
+__global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned short* z, long long stride, int n_all, int label_base0, int k,
+                                                             int parts, int have0, int have1, unsigned short* run_val, int* run_idx) {
   __shared__ unsigned hist[1024];
   __shared__ __attribute__((aligned(16))) unsigned sel_key[TOPK_MAX];
   __shared__ __attribute__((aligned(16))) int sel_idx[TOPK_MAX];
@@ -43,9 +48,14 @@ __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned shor
   __shared__ __attribute__((aligned(16))) int cand_idx[TOPK_CAP];   // index in the chunk (negative: an entry kept from earlier chunks)
   __shared__ unsigned s_bin, s_above, s_count, s_ncand, wtot[TOPK_NT / 64];
   const int tid = threadIdx.x;
-  const unsigned short* row = z + (size_t)blockIdx.x * stride;
-  unsigned short* rv = run_val + (size_t)blockIdx.x * TOPK_MAX;
-  int* ri = run_idx + (size_t)blockIdx.x * TOPK_MAX;
+  const int brow = parts == 2 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x, part = parts == 2 ? (int)(blockIdx.x & 1) : 0;
+  const int first = part == 0 ? 0 : topk_split(n_all);                      // this workgroup's range of the chunk
+  const int n = parts == 2 ? (part == 0 ? topk_split(n_all) : n_all - first) : n_all;
+  const int label_base = label_base0 + first;
+  const int have = part == 0 ? have0 : have1;
+  const unsigned short* row = z + (size_t)brow * stride + first;
+  unsigned short* rv = run_val + ((size_t)brow * 2 + part) * TOPK_MAX;
+  int* ri = run_idx + ((size_t)brow * 2 + part) * TOPK_MAX;
   const int total = n + have;
   const int kk = k < total ? k : total;
   const unsigned mykey = tid < have ? topk_key(rv[tid]) : 0u;   // this thread's entry of the running list
@@ -276,13 +286,38 @@ __global__ __launch_bounds__(TOPK_NT) void topk_chunk_kernel(const unsigned shor
   }
 }
 
-// copies the first k entries of the running lists to the outputs [batch][k]
-__global__ void topk_finish_kernel(const unsigned short* run_val, const int* run_idx, int batch, int k, unsigned short* out_val, int* out_idx) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= batch * k) return;
-  const int b = i / k, j = i - b * k;
-  out_val[i] = run_val[(size_t)b * TOPK_MAX + j];
-  out_idx[i] = run_idx[(size_t)b * TOPK_MAX + j];
+// merges the two sorted lists of every batch row (have0 and have1 entries valid, have0 + have1 >= k, all label ids
+// distinct) and writes the first k entries to the outputs [batch][k]: an entry's position is its index in its own list
+// plus the number of entries of the other list that come before it (value descending, label ascending).
+// One workgroup of 2 * TOPK_MAX threads per row.
+__global__ __launch_bounds__(2 * TOPK_MAX) void topk_finish_kernel(const unsigned short* run_val, const int* run_idx, int k, int have0,
+                                                                  int have1, unsigned short* out_val, int* out_idx) {
+  __shared__ __attribute__((aligned(16))) unsigned fkey[2][TOPK_MAX];
+  __shared__ __attribute__((aligned(16))) int fidx[2][TOPK_MAX];
+  const int b = blockIdx.x, list = threadIdx.x / TOPK_MAX, j = threadIdx.x - list * TOPK_MAX;
+  const int mine = list == 0 ? have0 : have1;
+  const bool valid = j < mine;
+  const unsigned short bits = valid ? run_val[((size_t)b * 2 + list) * TOPK_MAX + j] : (unsigned short)0;
+  const int idx = valid ? run_idx[((size_t)b * 2 + list) * TOPK_MAX + j] : 0x7FFFFFFF;
+  const unsigned key = valid ? topk_key(bits) : 0u;   // an entry that is not there comes before nothing
+  fkey[list][j] = key;
+  fidx[list][j] = idx;
+  __syncthreads();
+  if (!valid) return;
+  int pos = j;
+#pragma unroll 8
+  for (int o = 0; o < TOPK_MAX; o += 4) {
+    const uint4 ko = *(const uint4*)&fkey[list ^ 1][o];
+    const int4 io = *(const int4*)&fidx[list ^ 1][o];
+    pos += (ko.x > key || (ko.x == key && io.x < idx)) ? 1 : 0;
+    pos += (ko.y > key || (ko.y == key && io.y < idx)) ? 1 : 0;
+    pos += (ko.z > key || (ko.z == key && io.z < idx)) ? 1 : 0;
+    pos += (ko.w > key || (ko.w == key && io.w < idx)) ? 1 : 0;
+  }
+  if (pos < k) {
+    out_val[(size_t)b * k + pos] = bits;
+    out_idx[(size_t)b * k + pos] = idx;
+  }
 }
 
 }  // namespace xmc

@@ -83,7 +83,7 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one group of chunks (up to 2^17 labels, or one
- * chunk of up to 2^18 rows) and the running lists. */
+ * chunk of up to 2^18 rows) and the running lists (two of 128 entries per batch row). */
 size_t xmc_topk_scratch_bytes(int rows_per_chunk);
 
 /* Inference with the top-k taken chunk by chunk: what the evaluation loop computes as
