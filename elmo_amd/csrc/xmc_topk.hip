@@ -3,7 +3,8 @@
 // written to a chunk-sized buffer and reduced to the k best per batch row, so the [B, L] matrix (172 MB at B = 128,
 // L = 670 K) is never allocated.
 //
-// One workgroup per batch row.  Candidates = the k entries kept so far (from the chunks before, hence smaller label
+// One workgroup per batch row and list (a row has two lists: a large group of chunks is split between two workgroups,
+// and topk_finish_kernel merges the lists at the end).  Candidates = the k entries kept so far (from the chunks before, hence smaller label
 // ids) followed by the chunk's logits in label order.  Radix select on a 16-bit key that orders bf16 values (two passes
 // of 256 bins find the key T of the k-th largest), then everything above T is taken, entries equal to T are taken in
 // candidate order until k are full (ties go to the smaller label id: a second radix select, on the label, among the
@@ -17,7 +18,7 @@
 namespace xmc {
 
 constexpr int TOPK_MAX = 128;   // largest k
-constexpr int TOPK_NT = 1024;  // one workgroup per batch row: sixteen wavefronts keep enough loads in flight on its compute unit
+constexpr int TOPK_NT = 1024;  // sixteen wavefronts keep enough loads in flight on the workgroup's compute unit
 template <int N> struct TopkBins { static constexpr int value = N; };
 typedef TopkBins<256> B256;
 typedef TopkBins<1024> B1024;
