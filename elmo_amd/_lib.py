@@ -26,6 +26,7 @@ def load():
     lib = ctypes.CDLL(LIB_PATH)
     vp, i32, f32, sz, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_longlong
     lib.xmc_version.restype = i32
+    lib.xmc_source_hash.restype = ctypes.c_char_p
     lib.xmc_error_string.restype = ctypes.c_char_p
     lib.xmc_error_string.argtypes = [i32]
     lib.xmc_workspace_bytes.restype = sz

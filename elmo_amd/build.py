@@ -12,9 +12,25 @@ HIPCC_FLAGS = [
 ]
 
 
+def source_files():
+    csrc = os.path.join(HERE, "csrc")
+    return sorted(os.path.join(csrc, f) for f in os.listdir(csrc)) + [os.path.join(os.path.dirname(HERE), "include", "elmo_xmc.h")]
+
+
+def source_hash():
+    """Digest of the HIP sources and the header; the library reports the one it was built from (xmc_source_hash)."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in source_files():
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + [SRC, "-o", OUT]
+    cmd = [hipcc] + HIPCC_FLAGS + [f'-DXMC_SOURCE_HASH="{source_hash()}"', SRC, "-o", OUT]
     if verbose:
         cmd.append("-Rpass-analysis=kernel-resource-usage")
     res = subprocess.run(cmd, capture_output=True, text=True)

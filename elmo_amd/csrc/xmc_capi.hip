@@ -100,6 +100,11 @@ extern "C" {
 
 int xmc_version(void) { return 1; }
 
+#ifndef XMC_SOURCE_HASH
+#define XMC_SOURCE_HASH "unknown"
+#endif
+const char* xmc_source_hash(void) { return XMC_SOURCE_HASH; }
+
 const char* xmc_error_string(int status) {
   switch (status) {
     case XMC_OK: return "ok";

@@ -43,6 +43,9 @@ enum {
 };
 
 int xmc_version(void);
+/* Build aid (no counterpart in the reference): digest of the sources this library was compiled from, as
+ * elmo_amd/build.py computes it, or "unknown".  A test compares it with the sources in the tree. */
+const char* xmc_source_hash(void);
 const char* xmc_error_string(int status);
 
 /* Bytes of workspace the step needs for `num_chunks` chunks of `rows_per_chunk` rows (features fixed at 768).

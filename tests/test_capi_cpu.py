@@ -26,15 +26,12 @@ def test_every_declared_symbol_is_exported():
         assert hasattr(lib, n), n
 
 
-def test_library_is_not_older_than_its_sources():
+def test_library_was_built_from_the_sources_in_the_tree():
     """The GPU runs load the library that is in the tree: one that predates an edit of the sources would test and
-    measure the old kernels."""
-    lib_path = os.path.join(ROOT, "elmo_amd", "libelmo_xmc.so")
-    assert os.path.exists(lib_path)
-    csrc = os.path.join(ROOT, "elmo_amd", "csrc")
-    sources = [os.path.join(csrc, f) for f in os.listdir(csrc)] + [os.path.join(ROOT, "include", "elmo_xmc.h")]
-    newest = max(sources, key=os.path.getmtime)
-    assert os.path.getmtime(lib_path) >= os.path.getmtime(newest), f"{newest} is newer than the built library: rebuild it"
+    measure the old kernels.  The library carries a digest of the sources it was compiled from."""
+    from elmo_amd import build
+    built_from = _lib.load().xmc_source_hash().decode()
+    assert built_from == build.source_hash(), "the sources changed after the library was built: rebuild it"
 
 
 def test_version_and_error_strings():
