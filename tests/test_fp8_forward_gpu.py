@@ -47,6 +47,8 @@ def test_forward_scales(gpu):
     (2, 1024, 20, 2048, 128),       # batch padded to 32, largest k
     (4, 4096, 128, 16000, 100),     # full batch
     (2, 64, 16, 70, 70),            # k equal to the number of labels
+    (3, 16384, 32, 49000, 100),     # one group above 32,768 labels: two workgroups and two lists per batch row
+    (5, 16384, 16, 81920, 7),       # the same, k small, nothing dropped
 ])
 def test_topk_forward(gpu, nc, rows, batch, num_labels, k):
     """Chunk-wise top-k against the dense logits of the same library (bit-equal values, ids that point at them, the
@@ -86,18 +88,20 @@ def test_topk_with_repeated_values(gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("k", [100, 7])
-def test_topk_when_most_logits_tie(gpu, k):
+@pytest.mark.parametrize("k,nc", [(100, 2), (7, 2), (100, 3), (7, 3)])
+def test_topk_when_most_logits_tie(gpu, k, nc):
     """Nearly all rows of W are one and the same row: more logits reach the running bound than the selection keeps in
-    fast memory, and the k-th value is a tie of thousands that the label id has to break."""
+    fast memory, and the k-th value is a tie of thousands that the label id has to break - with three chunks across
+    the two lists of a batch row, which the last kernel merges."""
     from elmo_amd import ops
     rng = np.random.default_rng(11)
-    rows, nc = 16384, 2
+    rows = 16384
     base = rng.choice(np.array([0x30, 0xB0, 0x38, 0x28], dtype=np.uint8), size=768)
     codes = np.tile(base, (nc * rows, 1))
     odd = rng.choice(nc * rows, size=60, replace=False)                # a few rows that differ, above or below the rest
     codes[odd] = rng.choice(np.array([0x30, 0xB0, 0x38, 0x28], dtype=np.uint8), size=(60, 768))
-    case = dict(x=synth.make_x(24, 768, 6), chunks=[codes[:rows].copy(), codes[rows:].copy()], labels=np.zeros((0, 2), np.int32))
+    case = dict(x=synth.make_x(24, 768, 6), chunks=[codes[c * rows:(c + 1) * rows].copy() for c in range(nc)],
+                labels=np.zeros((0, 2), np.int32))
     chunks, x, _ = H.to_device_case(case, gpu)
     num_labels = nc * rows - 5
     dense = ops.fp8_forward(chunks, x, num_labels).float().cpu().numpy()
