@@ -51,7 +51,8 @@ constexpr int QG_PIECES = (BP * QPL_S + 1023) / 1024;   // wave-wide loads per G
 constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432), padded
 constexpr int QSLOTS = 8;                 // exchange slots per quad
 constexpr int QLDS_G = QRING * QWC_BYTES; // LDS offset of the two gathered-G buffers
-constexpr int QRS = D + 16;               // LDS row stride of the own-rows image (49 x 16 bytes)
+constexpr int QRS = D + 32;               // LDS row stride of the own-rows image (50 x 16 bytes: with an even number of
+                                          // 16-byte units per row the 16-byte operand reads of stage A have no bank conflicts)
 constexpr int QROW_BYTES = 13 * 1024;     // 16 rows x 784 = 12544, padded to 13 wave-wide loads
 constexpr int QRRING = 3;                 // own-rows images in flight
 constexpr int QGBUF = 2;                  // gathered-G buffers: in use, in flight
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   QT_DECL
   // Per-lane source rows and byte offsets of the wave-wide pieces this wavefront loads (pieces v and v+8 of an image).
   // own-column image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 pieces of 1 KiB
-  // own-rows image:   rows 16m..16m+15, 16 x 49 chunks of 16 bytes (48 data + 1 pad) = 13 pieces
+  // own-rows image:   rows 16m..16m+15, 16 x 50 chunks of 16 bytes (48 data + 2 pad) = 13 pieces
   // The byte offsets are kept per lane for full tiles (nearly all): issuing a piece then costs no vector instruction.
   // A tile cut short by the end of its chunk recomputes them with the row clamped to the last valid one.
   auto wcol_offset = [&](int s, int last_row) {
@@ -322,8 +323,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     return (unsigned)(min(wr, last_row) * D + QCOLS * m + min(ch - wr * 13, 11) * 16);
   };
   auto rows_offset = [&](int s, int last_row) {
-    const int ch = (v + 8 * s) * 64 + lane, rr = ch / 49;
-    return (unsigned)(min(16 * m + min(rr, 15), last_row) * D + min(ch - rr * 49, 47) * 16);
+    const int ch = (v + 8 * s) * 64 + lane, rr = ch / (QRS / 16);
+    return (unsigned)(min(16 * m + min(rr, 15), last_row) * D + min(ch - rr * (QRS / 16), 47) * 16);
   };
   unsigned woff_full[2], roff_full[2];
 #pragma unroll
@@ -365,13 +366,14 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   auto stage_a = [&](int i, int slot, const QTile& q) {
     floatx4 z = floatx4{0.f, 0.f, 0.f, 0.f};
     {
-      // lane (row l16, k group kg) holds 32 consecutive bytes per K step
-      const unsigned asrc = (unsigned)(QLDS_R + slot * QROW_BYTES) + l16 * QRS + kg * 32;
+      // lane (row l16, k group kg) holds bytes 16kg..16kg+15 and 64+16kg..64+16kg+15 of every 128-byte K step (the X
+      // image is built in the same order): two 16-byte reads whose lanes tile the LDS banks
+      const unsigned asrc = (unsigned)(QLDS_R + slot * QROW_BYTES) + l16 * QRS + kg * 16;
       // the reads of three K steps are in flight at a time
       intx4 alo[6], ahi[6];
       auto rd = [&](int ks) {
         alo[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128);
-        ahi[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128 + 16);
+        ahi[ks] = *(const __attribute__((address_space(3))) intx4*)(lds + asrc + ks * 128 + 64);
       };
       rd(0); rd(1); rd(2);
       QFENCE();
@@ -677,7 +679,8 @@ __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* 
   packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v[0]), clamp448(v[1]), packed, false);
   packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v[2]), clamp448(v[3]), packed, true);
   {
-    int ks = k >> 7, kgq = (k >> 5) & 3, jq = k & 31;
+    // K step ks of 128 features; within it lane group kgq holds features 16kgq..16kgq+15 and 64+16kgq..64+16kgq+15
+    int ks = k >> 7, pk = k & 127, kgq = (pk >> 4) & 3, jq = ((pk >> 6) << 4) | (pk & 15);
     size_t off = ((size_t)(((b >> 4) * 6 + ks) * 64 + ((b & 15) + 16 * kgq))) * 32 + jq;
     *(int*)(xq + off) = packed;
   }
