@@ -590,6 +590,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         const int nbg = 2 * h + nb;
         const int row = 16 * nbg + l16;
         unsigned outw[3];
+        float t[3][4];
 #pragma unroll
         for (int cg = 0; cg < 3; cg++) {
           floatx4 a = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -597,10 +598,39 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
           for (int ks = 0; ks < 4; ks++) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][ks], bg[nb][ks], a, 0, 0, 0);
           const unsigned wv = wq[nb][cg];
           floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, true);
-          float t0 = __builtin_fmaf(-p.lr_eff, a[0], w01.x), t1 = __builtin_fmaf(-p.lr_eff, a[1], w01.y);
-          float t2 = __builtin_fmaf(-p.lr_eff, a[2], w23.x), t3 = __builtin_fmaf(-p.lr_eff, a[3], w23.y);
-          outw[cg] = round4<MODE>(t0, t1, t2, t3, (unsigned)(q.row0 + row), grow0 + 16 * nbg,
-                                  (unsigned)(QCOLS * m + 48 * fg + 12 * kg + 4 * cg), q.seed);
+          t[cg][0] = __builtin_fmaf(-p.lr_eff, a[0], w01.x); t[cg][1] = __builtin_fmaf(-p.lr_eff, a[1], w01.y);
+          t[cg][2] = __builtin_fmaf(-p.lr_eff, a[2], w23.x); t[cg][3] = __builtin_fmaf(-p.lr_eff, a[3], w23.y);
+        }
+        if (MODE == ROUND_SR_FAST) {
+          // The converter does not saturate.  Results beyond +-448 are rare: the twelve values of a lane are clamped
+          // only if some lane of the wavefront has one (six max3 and a compare instead of twelve med3).
+          float mx = 0.f;
+#pragma unroll
+          for (int cg = 0; cg < 3; cg++)
+            mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(t[cg][0]), __builtin_fabsf(t[cg][1])),
+                                                     __builtin_fmaxf(__builtin_fabsf(t[cg][2]), __builtin_fabsf(t[cg][3]))));
+          if (__builtin_amdgcn_ballot_w64(!(mx <= 448.0f)) != 0) {
+#pragma unroll
+            for (int cg = 0; cg < 3; cg++)
+#pragma unroll
+              for (int e = 0; e < 4; e++) t[cg][e] = clamp448(t[cg][e]);
+          }
+#pragma unroll
+          for (int cg = 0; cg < 3; cg++) {
+            const unsigned hsh = fast_mix((grow0 + 16 * nbg) * (unsigned)(D / 4) + (unsigned)((QCOLS * m + 48 * fg + 12 * kg + 4 * cg) >> 2), q.seed);
+            int packed;
+            asm volatile("" : "=v"(packed));   // every byte is written below
+            packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[cg][0], fast_word(hsh, 0), packed, 0);
+            packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[cg][1], fast_word(hsh, 1), packed, 1);
+            packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[cg][2], fast_word(hsh, 2), packed, 2);
+            packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[cg][3], fast_word(hsh, 3), packed, 3);
+            outw[cg] = (unsigned)packed;
+          }
+        } else {
+#pragma unroll
+          for (int cg = 0; cg < 3; cg++)
+            outw[cg] = round4<MODE>(t[cg][0], t[cg][1], t[cg][2], t[cg][3], (unsigned)(q.row0 + row), grow0 + 16 * nbg,
+                                    (unsigned)(QCOLS * m + 48 * fg + 12 * kg + 4 * cg), q.seed);
         }
         if (row < q.rows_valid) {
           // the pointer comes out of scalar registers as an integer: say that it is global memory, or the store
