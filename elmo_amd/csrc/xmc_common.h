@@ -73,15 +73,15 @@ __device__ __forceinline__ unsigned philox_word0(unsigned off, unsigned k0, unsi
   return c0;
 }
 
-// Counter hash of the fast stochastic-rounding mode: one 32-bit mix per 4 consecutive weights of a row,
-// expanded to four words by odd multipliers.  idx = global_row * (D/4) + col/4.
+// Counter hash of the fast stochastic-rounding mode: one 32-bit mix per 4 consecutive weights of a row; the first
+// weight takes the mix itself, the other three its products with odd constants.  idx = global_row * (D/4) + col/4.
 __device__ __forceinline__ unsigned fast_mix(unsigned idx, unsigned seed) {
   unsigned h = idx * 0x9E3779B1u + seed;
   h ^= h >> 16; h *= 0x85EBCA77u; h ^= h >> 15;
   return h;
 }
 __device__ __forceinline__ unsigned fast_word(unsigned h, int i) {
-  const unsigned k[4] = {0xC2B2AE3Du, 0x27D4EB2Fu, 0x165667B1u, 0x9E3779B1u};
+  const unsigned k[4] = {1u, 0x27D4EB2Fu, 0x165667B1u, 0x9E3779B1u};
   return h * k[i];
 }
 

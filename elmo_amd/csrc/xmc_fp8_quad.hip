@@ -606,9 +606,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
           // only if some lane of the wavefront has one (six max3 and a compare instead of twelve med3).
           float mx = 0.f;
 #pragma unroll
-          for (int cg = 0; cg < 3; cg++)
-            mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(t[cg][0]), __builtin_fabsf(t[cg][1])),
-                                                     __builtin_fmaxf(__builtin_fabsf(t[cg][2]), __builtin_fabsf(t[cg][3]))));
+          for (int cg = 0; cg < 3; cg++) {
+            mx = __builtin_fmaxf(__builtin_fmaxf(mx, __builtin_fabsf(t[cg][0])), __builtin_fabsf(t[cg][1]));
+            mx = __builtin_fmaxf(__builtin_fmaxf(mx, __builtin_fabsf(t[cg][2])), __builtin_fabsf(t[cg][3]));
+          }
           if (__builtin_amdgcn_ballot_w64(!(mx <= 448.0f)) != 0) {
 #pragma unroll
             for (int cg = 0; cg < 3; cg++)

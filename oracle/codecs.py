@@ -198,13 +198,13 @@ def sr_e4m3_exact(t, rand32):
 # --------------------------------------------------------------------------- this build's fast SR random words
 def fast_sr_words(seed, global_rows, cols, features=768):
     """Random word per weight of the fast stochastic-rounding mode (not part of the reference): one 32-bit mix per
-    group of 4 consecutive weights of a row, idx = global_row * (features/4) + col/4, expanded to four words by
-    odd multipliers.  Restates fast_mix/fast_word of elmo_amd/csrc/xmc_common.h."""
+    group of 4 consecutive weights of a row, idx = global_row * (features/4) + col/4; the first weight takes the mix
+    itself, the other three its products with odd constants.  Restates fast_mix/fast_word of elmo_amd/csrc/xmc_common.h."""
     M = np.uint64(0xFFFFFFFF)
     idx = (np.asarray(global_rows, dtype=np.uint64) * np.uint64(features // 4) + (np.asarray(cols, dtype=np.uint64) >> np.uint64(2))) & M
     h = (idx * np.uint64(0x9E3779B1) + np.uint64(int(seed) & 0xFFFFFFFF)) & M
     h ^= h >> np.uint64(16)
     h = (h * np.uint64(0x85EBCA77)) & M
     h ^= h >> np.uint64(15)
-    k = np.array([0xC2B2AE3D, 0x27D4EB2F, 0x165667B1, 0x9E3779B1], dtype=np.uint64)[np.asarray(cols, dtype=np.int64) & 3]
+    k = np.array([1, 0x27D4EB2F, 0x165667B1, 0x9E3779B1], dtype=np.uint64)[np.asarray(cols, dtype=np.int64) & 3]
     return ((h * k) & M).astype(np.uint32)
