@@ -400,14 +400,29 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     if (q.p1 > q.p0) {
       float sg[4] = {__uint_as_float(sb[0] << 16), __uint_as_float(sb[0] & 0xFFFF0000u), __uint_as_float(sb[1] << 16),
                      __uint_as_float(sb[1] & 0xFFFF0000u)};
-      for (int e = q.p0; e < q.p1; e++) {
-        const unsigned key = ckeys[e];
-        const unsigned prev = e > 0 ? ckeys[e - 1] : ~key;
-        const unsigned l = (key >> 8) - q.label0 - (unsigned)r0;
-        const bool mine = prev != key && l < 4u && (key & 255u) == (unsigned)(16 * v + l16);
+      // The keys come eight at a time through the scalar path (one wait per eight; the first tiles of a chunk sorted
+      // by label frequency hold hundreds of positives), and a key costs vector instructions only if it lies in this
+      // wavefront's block (label rows 16m.., batch rows 16v..).  Up to seven keys behind the tile's last are read and
+      // ignored; the buffer behind the keys belongs to the workspace.
+      typedef unsigned q_keysx8 __attribute__((ext_vector_type(8), aligned(4)));
+      const unsigned lbase = q.label0 + 16u * (unsigned)m;
+      unsigned prev = q.p0 > 0 ? ckeys[q.p0 - 1] : ~ckeys[q.p0];
+      for (int e0 = q.p0; e0 < q.p1; e0 += 8) {
+        const q_keysx8 kk = *(const __attribute__((address_space(4))) q_keysx8*)(ckeys + e0);
 #pragma unroll
-        for (int q4 = 0; q4 < 4; q4++)
-          if (mine && l == (unsigned)q4) sg[q4] = bf16_rt(sg[q4] - 1.0f);
+        for (int j = 0; j < 8; j++) {
+          const unsigned key = kk[j];
+          const unsigned lrel = (key >> 8) - lbase;   // label row within this member's sixteen
+          if (e0 + j < q.p1 && key != prev && lrel < 16u && ((key >> 4) & 15u) == (unsigned)v) {
+            const bool mine = (unsigned)kg == (lrel >> 2) && (unsigned)l16 == (key & 15u);
+            const unsigned q4 = lrel & 3u;   // wave-uniform: one of the lane's four labels
+            if (q4 == 0u) sg[0] = mine ? bf16_rt(sg[0] - 1.0f) : sg[0];
+            else if (q4 == 1u) sg[1] = mine ? bf16_rt(sg[1] - 1.0f) : sg[1];
+            else if (q4 == 2u) sg[2] = mine ? bf16_rt(sg[2] - 1.0f) : sg[2];
+            else sg[3] = mine ? bf16_rt(sg[3] - 1.0f) : sg[3];
+          }
+          prev = key;
+        }
       }
       sb[0] = bf16_pack2(sg[0], sg[1]);
       sb[1] = bf16_pack2(sg[2], sg[3]);
