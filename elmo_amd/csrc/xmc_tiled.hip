@@ -193,36 +193,53 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
     }
     // acc[lb][e] = Z[label 32 st + 16 lb + 4kg + e][batch 16v + l16]
     float lsum = 0.f;
+    float sg[2][4], zf[2][4];
 #pragma unroll
     for (int lb = 0; lb < 2; lb++) {
       const int r0 = st * TLG_ROWS + 16 * lb;
-      float sg[4], zf[4];
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        zf[e] = bf16_rt(acc[lb][e]);
-        sg[e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf[e] * nlog2e)));
+        zf[lb][e] = bf16_rt(acc[lb][e]);
+        sg[lb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf[lb][e] * nlog2e)));
         if (LOSS && r0 + 4 * kg + e < rows && (int)brow0 + 16 * v + l16 < batch)
-          lsum += __builtin_fmaxf(zf[e], 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf[e]) * 1.44269504088896340736f));
+          lsum += __builtin_fmaxf(zf[lb][e], 0.f) + 0.69314718055994530942f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fabsf(zf[lb][e]) * 1.44269504088896340736f));
       }
-      // positives of the enclosing 64-row tile (set semantics: a repeated key counts once)
-      const unsigned lbase = label0_chunk + (unsigned)(r0 + 4 * kg);
-      for (int e = p0; e < p1; e++) {
-        const unsigned key = ckeys[e];
-        const unsigned prev = e > 0 ? ckeys[e - 1] : ~key;
-        const unsigned l = (key >> 8) - lbase;
-        const unsigned b = (key & 255u) - brow0;   // batch row within this half
-        if (prev != key && l < 4u && b == (unsigned)(16 * v + l16)) {
+    }
+    // Positives of the enclosing 64-row tile (set semantics: a repeated key counts once).  The keys come eight at a time
+    // through the scalar path (the first tiles of a chunk sorted by label frequency hold hundreds), and a key costs vector
+    // instructions only if it lies in this wavefront's block (the sub-tile's 32 labels, batch rows 16v.. of this half).
+    // Up to seven keys behind the tile's last are read and ignored; the buffer behind the keys belongs to the workspace.
+    if (p1 > p0) {
+      typedef unsigned t_keysx8 __attribute__((ext_vector_type(8), aligned(4)));
+      const unsigned lbase = label0_chunk + (unsigned)(st * TLG_ROWS);
+      unsigned prev = p0 > 0 ? ckeys[p0 - 1] : ~ckeys[p0];
+      for (int e0 = p0; e0 < p1; e0 += 8) {
+        const t_keysx8 kk = *(const __attribute__((address_space(4))) t_keysx8*)(ckeys + e0);
 #pragma unroll
-          for (int q4 = 0; q4 < 4; q4++)
-            if (l == (unsigned)q4) {
-              sg[q4] = bf16_rt(sg[q4] - 1.0f);
-              if (LOSS && r0 + 4 * kg + q4 < rows) lsum -= zf[q4];
-            }
+        for (int j = 0; j < 8; j++) {
+          const unsigned key = kk[j];
+          const unsigned lrel = (key >> 8) - lbase;      // label within the sub-tile
+          const unsigned b = (key & 255u) - brow0;       // batch row within this half
+          if (e0 + j < p1 && key != prev && lrel < (unsigned)TLG_ROWS && (b >> 4) == (unsigned)v) {
+            const bool mine = (unsigned)kg == ((lrel >> 2) & 3u) && (unsigned)l16 == (b & 15u);
+            const unsigned sel = ((lrel >> 4) << 2) | (lrel & 3u);   // wave-uniform: label block and one of the lane's four labels
+#pragma unroll
+            for (int c = 0; c < 8; c++)
+              if (sel == (unsigned)c) {
+                if (LOSS && st * TLG_ROWS + 16 * (c >> 2) + 4 * kg + (c & 3) < rows) lsum -= mine ? zf[c >> 2][c & 3] : 0.f;
+                sg[c >> 2][c & 3] = mine ? bf16_rt(sg[c >> 2][c & 3] - 1.0f) : sg[c >> 2][c & 3];
+              }
+          }
+          prev = key;
         }
       }
+    }
+#pragma unroll
+    for (int lb = 0; lb < 2; lb++) {
+      const int r0 = st * TLG_ROWS + 16 * lb;
       unsigned short sb[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[e]) : (unsigned short)0;
+      for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[lb][e]) : (unsigned short)0;
       uint2 o;
       o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
       o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
