@@ -323,7 +323,8 @@ def main():
             traffic = json.load(f).get(f"{kernel_name}:{cfg.name}:{args.round}")
 
     out = {
-        "metric": "XMC classifier train steps/sec at 670K labels FP8",
+        "metric": "XMC classifier train steps/sec at 670K labels FP8" if cfg.name == "cfg2_fp8_670k" else
+                  "XMC classifier train steps/sec at %d labels FP8" % cfg.num_labels,
         "value": steps_per_s, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3 weights+logits MFMA, bf16 gradient MFMA, fp32 accumulate", "data": "synthetic",
