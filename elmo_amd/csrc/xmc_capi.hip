@@ -162,7 +162,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     StepParams p;
     for (int c = 0; c < MAX_CHUNKS; c++) {
       p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
-      p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+      p.seed[c] = (c < num_chunks && seeds) ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c]) : seeds[c]) : 0u;
     }
     p.num_chunks = num_chunks;
     p.rows_per_chunk = rows_per_chunk;
@@ -191,7 +191,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     QuadParams p;
     for (int c = 0; c < MAX_CHUNKS; c++) {
       p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
-      p.seed[c] = (c < num_chunks && seeds) ? seeds[c] : 0u;
+      p.seed[c] = (c < num_chunks && seeds) ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c]) : seeds[c]) : 0u;
     }
     p.num_chunks = num_chunks;
     p.rows_per_chunk = rows_per_chunk;
@@ -417,7 +417,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int rp = (rows + TL - 1) / TL * TL;           // padded rows of this chunk (G buffers use the stride rows_pad)
     const int tiles = rp / TL;
     const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;
-    const unsigned seed = seeds ? seeds[c] : 0u;
+    const unsigned seed = seeds ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c]) : seeds[c]) : 0u;
     const int nh = c == 0 ? num_head : 0;   // the compensated head lives in chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127)
     int range = (rp + T_SPLITS - 1) / T_SPLITS;
     range = (range + TL - 1) / TL * TL;

@@ -75,6 +75,12 @@ __device__ __forceinline__ unsigned philox_word0(unsigned off, unsigned k0, unsi
 
 // Counter hash of the fast stochastic-rounding mode: one 32-bit mix per 4 consecutive weights of a row; the first
 // weight takes the mix itself, the other three its products with odd constants.  idx = global_row * (D/4) + col/4.
+// The caller's seed goes through a full 32-bit mixer once, on the host, before it reaches fast_mix: seeds that differ
+// in a few bits (s and s + 1, say) must not give related words.
+__host__ __device__ inline unsigned fast_seed(unsigned s) {
+  s ^= s >> 16; s *= 0x7FEB352Du; s ^= s >> 15; s *= 0x846CA68Bu; s ^= s >> 16;
+  return s;
+}
 __device__ __forceinline__ unsigned fast_mix(unsigned idx, unsigned seed) {
   unsigned h = idx * 0x9E3779B1u + seed;
   h ^= h >> 16; h *= 0x85EBCA77u; h ^= h >> 15;

@@ -199,10 +199,13 @@ def sr_e4m3_exact(t, rand32):
 def fast_sr_words(seed, global_rows, cols, features=768):
     """Random word per weight of the fast stochastic-rounding mode (not part of the reference): one 32-bit mix per
     group of 4 consecutive weights of a row, idx = global_row * (features/4) + col/4; the first weight takes the mix
-    itself, the other three its products with odd constants.  Restates fast_mix/fast_word of elmo_amd/csrc/xmc_common.h."""
+    itself, the other three its products with odd constants; the seed is mixed first.  Restates
+    fast_seed/fast_mix/fast_word of elmo_amd/csrc/xmc_common.h."""
     M = np.uint64(0xFFFFFFFF)
     idx = (np.asarray(global_rows, dtype=np.uint64) * np.uint64(features // 4) + (np.asarray(cols, dtype=np.uint64) >> np.uint64(2))) & M
-    h = (idx * np.uint64(0x9E3779B1) + np.uint64(int(seed) & 0xFFFFFFFF)) & M
+    sd = int(seed) & 0xFFFFFFFF            # fast_seed: the caller's seed through a full 32-bit mixer
+    sd ^= sd >> 16; sd = (sd * 0x7FEB352D) & 0xFFFFFFFF; sd ^= sd >> 15; sd = (sd * 0x846CA68B) & 0xFFFFFFFF; sd ^= sd >> 16
+    h = (idx * np.uint64(0x9E3779B1) + np.uint64(sd)) & M
     h ^= h >> np.uint64(16)
     h = (h * np.uint64(0x85EBCA77)) & M
     h ^= h >> np.uint64(15)

@@ -82,6 +82,7 @@ def test_argument_validation_without_a_device():
     assert status(mode=2, seeds=None) == -1
     assert status(sw=0.0) == -2 and status(sx=-1.0) == -2
     assert status(labels=None, nnz=3) == -1
+    assert status(labels=P + 4) == -3          # the (row, label) pairs are read whole: 8-byte alignment
 
 
 def test_python_wrapper_raises_on_error_status():

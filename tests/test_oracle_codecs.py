@@ -162,3 +162,28 @@ def test_e5m2_codec_matches_torch():
     assert np.array_equal(C.e5m2_encode(x, saturate=False), ref_codes)                  # overflow -> inf as torch
     big = np.array([61440.0, 1e6, np.inf, -1e9], dtype=np.float32)
     assert np.array_equal(C.e5m2_decode(C.e5m2_encode(big, saturate=True)), np.array([57344.0, 57344.0, 57344.0, -57344.0], np.float32))
+
+
+def test_fast_rounding_words_look_uniform_and_independent():
+    """The random words of the fast rounding mode (this build's own definition: one hash per four weights, the first
+    weight takes it as it is, the others multiples of it): the top bits, which the converter uses, are uniform for every
+    position in the group, and neighbouring weights, rows and seeds are uncorrelated."""
+    rows = np.arange(4096, dtype=np.int64)[:, None]
+    cols = np.arange(768, dtype=np.int64)[None, :]
+    w = C.fast_sr_words(12345, np.broadcast_to(rows, (4096, 768)), np.broadcast_to(cols, (4096, 768)))
+    u = (w >> np.uint32(12)).astype(np.float64) / float(1 << 20)        # the 20 bits above the discarded ones
+    n = u.size
+    for pos in range(4):                                                # every position of the group of four
+        v = u[:, pos::4]
+        assert abs(v.mean() - 0.5) < 4.0 / np.sqrt(12 * v.size)
+        hist = np.bincount((v * 16).astype(np.int64).ravel(), minlength=16)
+        assert np.abs(hist / v.size - 1 / 16).max() < 5.0 * np.sqrt((1 / 16) * (15 / 16) / v.size)
+    def corr(a, b):
+        return float(np.corrcoef(a.ravel(), b.ravel())[0, 1])
+    lim = 5.0 / np.sqrt(n / 4)
+    assert abs(corr(u[:, 0::4], u[:, 1::4])) < lim and abs(corr(u[:, 0::4], u[:, 3::4])) < lim      # within a group
+    assert abs(corr(u[:, 1::4], u[:, 2::4])) < lim
+    assert abs(corr(u[:, :-4], u[:, 4:])) < 5.0 / np.sqrt(n) and abs(corr(u[:-1], u[1:])) < 5.0 / np.sqrt(n)   # next group, next row
+    w2 = C.fast_sr_words(12346, np.broadcast_to(rows, (4096, 768)), np.broadcast_to(cols, (4096, 768)))
+    u2 = (w2 >> np.uint32(12)).astype(np.float64) / float(1 << 20)
+    assert abs(corr(u, u2)) < 5.0 / np.sqrt(n)                                                      # next seed
