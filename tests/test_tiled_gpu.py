@@ -398,3 +398,38 @@ def test_head_kahan_module(gpu):
     cfg2.training.FP8 = types.SimpleNamespace(using_head_kahan=False, fp8_head_kahan=False, head_ratio=0.2)
     plain = Fp8XMCBCEChunkedHeadKahanLayer(cfg2)                      # no buffer: the fused kernel
     assert plain.xfc_forward_backward(tokens, labels, [0.05]) == 0 and not hasattr(plain, "head_kahan")
+
+
+def test_tiled_step_replays_in_a_captured_graph(gpu):
+    """The three-kernel path launches kernels only (no memset, no allocation, no synchronisation), so a caller may record
+    it into a graph: three replays, with eager work and synchronisations between them, give bit for bit what three eager
+    steps give (bf16 layer, round-to-nearest, ragged chunks, batch in two halves)."""
+    import torch
+    from elmo_amd import ops
+    x, w, labels = bf16_case(3000, 200, 36)
+    L, nc = w.shape[0], 2
+    cs = (L + nc - 1) // nc
+    wt = torch.from_numpy(C.bf16_bits(w).view(np.int16)).to(gpu).view(torch.bfloat16)
+    start = wt.clone()
+    views = [wt[c * cs:min((c + 1) * cs, L)] for c in range(nc)]
+    xt = torch.from_numpy(C.bf16_bits(x).view(np.int16)).to(gpu).view(torch.bfloat16)
+    lab = torch.from_numpy(labels).to(gpu).contiguous()
+    ws = ops.alloc_tiled_workspace(nc, cs, gpu, 200)
+    gout = torch.empty(200, 768, dtype=torch.bfloat16, device=gpu)
+    eager = []
+    for _ in range(3):
+        ops.tiled_step(views, cs, "bf16", xt, lab, 0.05, round_mode="rtn", workspace=ws, grad_out=gout)
+        eager.append((wt.view(torch.int16).clone(), gout.view(torch.int16).clone()))
+    wt.copy_(start)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.tiled_step(views, cs, "bf16", xt, lab, 0.05, round_mode="rtn", workspace=ws, grad_out=gout)
+    assert torch.equal(wt.view(torch.int16), start.view(torch.int16))      # the capture ran nothing
+    for k in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(wt.view(torch.int16), eager[k][0]), f"weights differ after replay {k}"
+        assert torch.equal(gout.view(torch.int16), eager[k][1]), f"grad_input differs after replay {k}"
+        scratch = torch.randn(1 << 20, device=gpu).sum().item()      # unrelated eager work between the replays
+        assert scratch == scratch
