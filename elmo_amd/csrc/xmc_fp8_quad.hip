@@ -707,7 +707,8 @@ __global__ __launch_bounds__(128) void reduce_gx_quad_kernel(const floatx4* part
 
 // Operand images of X for the quad kernel.
 //   xq: e4m3(X / scale_x) in v_mfma 16x16x128 B-operand order: operand index ((b/16)*6 + ks), lane = (b%16) + 16*kg,
-//       byte j: Xq[b][k = 128ks + 32kg + j]
+//       bytes 0..15: Xq[b][k = 128ks + 16kg + j], bytes 16..31: Xq[b][k = 128ks + 64 + 16kg + (j - 16)] (the order in which
+//       stage A reads the weight rows from LDS)
 //   xt: bf16 X^T in v_mfma 16x16x32 A-operand order: [((col/48)*3 + cg)*4 + ks][lane][8 bf16], lane = r + 16*kg,
 //       element j = X[32ks + 8kg + j][col] with col = 48*(col/48) + 12*(r/4) + 4*cg + r%4
 __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
