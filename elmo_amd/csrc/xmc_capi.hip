@@ -32,6 +32,8 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
     (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
     (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
+    (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 2>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
@@ -434,14 +436,22 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       if (weight_type == W_BF16) {
         if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        tiled_gradx_kernel<W_BF16><<<4 * splits, 256, TgxGeom<W_BF16>::LDS, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       } else {
         if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
         else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        tiled_gradx_kernel<W_E4M3><<<4 * splits, 256, TgxGeom<W_E4M3>::LDS, stream>>>(w, rows, rows_pad, rp, range, gb, partial);
       }
-      tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     }
+    // grad_X of the chunk: one pass over W for both batch halves, then the fixed-order sums per half
+    const size_t part_half = (size_t)T_SPLITS * 4 * 24 * 256;   // floatx4 elements of one half's partials
+    if (weight_type == W_BF16) {
+      if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * splits, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
+      else tiled_gradx_kernel<W_BF16, 2><<<4 * splits, 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
+    } else {
+      if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * splits, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
+      else tiled_gradx_kernel<W_E4M3, 2><<<4 * splits, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
+    }
+    for (int hh = 0; hh < halves; hh++)
+      tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial + (size_t)hh * part_half, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
     const int ugrid = 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
   tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, 256 * HV, (size_t)TUP_XBYTES * HV, stream>>>(                             \

@@ -27,8 +27,8 @@ constexpr size_t TW_XB = 0;                                        // X   [halve
 constexpr size_t TW_XT = TW_XB + (size_t)T_HALVES * BP * D * 2;    // X^T [halves][768][128] bf16
 constexpr size_t TW_KEYS = TW_XT + (size_t)T_HALVES * BP * D * 2;  // sorted positive keys
 constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [halves*128][768]
-constexpr size_t TW_PART = TW_GX + (size_t)T_HALVES * BP * D * 4;  // grad_X partials [T_SPLITS][128*768] fp32 (one half at a time)
-constexpr size_t TW_G = TW_PART + (size_t)T_SPLITS * BP * D * 4;   // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr
+constexpr size_t TW_PART = TW_GX + (size_t)T_HALVES * BP * D * 4;  // grad_X partials [halves][T_SPLITS][128*768] fp32
+constexpr size_t TW_G = TW_PART + (size_t)T_HALVES * T_SPLITS * BP * D * 4;   // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr
 
 __device__ __forceinline__ bf16x8 t_fp8x8_to_bf16x8(intx2 raw) {
   bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
@@ -291,32 +291,36 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
 //      8 KiB of G^T in operand order go straight to LDS, two steps ahead, in a ring of three stages; a compute unit's
 //      memory path handles few cache lines per clock, and register loads in operand order touched four times as many.
 //      The W operand comes back transposed (ds_read_b64_tr_b8 + exact fp8->bf16, or ds_read_b64_tr_b16).
-template <int WT> struct TgxGeom {
+//      With two batch halves (HV = 2) one pass over W serves both: the step's G^T of either half is staged, the W
+//      operand is read and converted once, and every wavefront keeps the accumulators of both halves.
+template <int WT, int HV> struct TgxGeom {
   static constexpr int ROWB = WT == W_BF16 ? 384 : 192;                  // bytes of this workgroup's features in one row
   static constexpr int STRIDE = ROWB + 16;                                // LDS row stride
   static constexpr int SLOTS = STRIDE / 16;                               // 16-byte slots per LDS row, the last one padding
   static constexpr int WPIECES = (32 * SLOTS + 63) / 64;                  // wave-wide loads of the W slice (7 or 13)
-  static constexpr int PIECES = WPIECES + 8;                              // ... and of G^T
+  static constexpr int PIECES = WPIECES + 8 * HV;                         // ... and of G^T (8 per batch half)
   static constexpr int PER_WAVE = (PIECES + 3) / 4;                       // every wavefront issues this many per step (4 or 6)
   static constexpr int WBYTES = WPIECES * 1024;
-  static constexpr int STAGE = WBYTES + 8192;
+  static constexpr int STAGE = WBYTES + 8192 * HV;
   static constexpr int LDS = 3 * STAGE;
 };
 
-template <int WT>
+template <int WT, int HV>
 __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, const unsigned short* gbl,
-                                                          floatx4* partial) {
-  typedef TgxGeom<WT> G;
+                                                          size_t g_half, floatx4* partial, size_t part_half) {
+  typedef TgxGeom<WT, HV> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
   const unsigned lds0 = (unsigned)(size_t)lds;
   const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fb = blockIdx.x & 3, split = blockIdx.x >> 2;
-  floatx4 acc[8][3];
+  floatx4 acc[HV][8][3];
 #pragma unroll
-  for (int mb = 0; mb < 8; mb++)
+  for (int hv = 0; hv < HV; hv++)
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+      for (int nn = 0; nn < 3; nn++) acc[hv][mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lbeg = split * range, lend = min(lbeg + range, bound);   // bound: this chunk's rows rounded up to a tile
   const int nsteps = lend > lbeg ? (lend - lbeg + 31) >> 5 : 0;
   // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv+4, ...; indices past the last piece repeat it),
@@ -332,8 +336,8 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
         t_lds_load16((const unsigned char*)w + ((size_t)lr * D + 192 * fb) * (WT == W_BF16 ? 2 : 1) + 16 * c16,
                      lds0 + (unsigned)(stage * G::STAGE + piece * 1024));
       } else {
-        const int gp = piece - G::WPIECES;
-        t_lds_load16((const unsigned char*)(gbl + ((size_t)((l0 >> 5) * 8 + gp) * 64 + lane) * 8),
+        const int gp = piece - G::WPIECES;   // piece gp & 7 of batch half gp >> 3
+        t_lds_load16((const unsigned char*)(gbl + (size_t)(gp >> 3) * g_half + ((size_t)((l0 >> 5) * 8 + (gp & 7)) * 64 + lane) * 8),
                      lds0 + (unsigned)(stage * G::STAGE + G::WBYTES + gp * 1024));
       }
     }
@@ -352,6 +356,11 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
     bf16x8 ga[8];
 #pragma unroll
     for (int mb = 0; mb < 8; mb++) ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + (mb * 64 + lane) * 16);
+    bf16x8 gh[HV == 2 ? 8 : 1];
+    if (HV == 2) {
+#pragma unroll
+      for (int mb = 0; mb < 8; mb++) gh[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + 8192 + (mb * 64 + lane) * 16);
+    }
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
@@ -369,16 +378,26 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
 #pragma unroll
     for (int mb = 0; mb < 8; mb++)
 #pragma unroll
-      for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
+      for (int nn = 0; nn < 3; nn++) acc[0][mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[0][mb][nn], 0, 0, 0);
+    if (HV == 2) {
+#pragma unroll
+      for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+        for (int nn = 0; nn < 3; nn++)
+          acc[HV - 1][mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gh[mb], wb[nn], acc[HV - 1][mb][nn], 0, 0, 0);
+    }
     stage = stage == 2 ? 0 : stage + 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end still target LDS
   // acc[mb][nn][e] = C[batch 16mb + 4kg + e][feature f0 + 16nn + l16]
-  floatx4* dst = partial + ((size_t)split * 4 + fb) * 24 * 256;
 #pragma unroll
-  for (int mb = 0; mb < 8; mb++)
+  for (int hv = 0; hv < HV; hv++) {
+    floatx4* dst = partial + (size_t)hv * part_half + ((size_t)split * 4 + fb) * 24 * 256;
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + tid] = acc[mb][nn];
+    for (int mb = 0; mb < 8; mb++)
+#pragma unroll
+      for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + tid] = acc[hv][mb][nn];
+  }
 }
 
 // sum of the partials of one chunk in a fixed order; bf16 weights: the chunk's contribution is rounded to bf16 before it
