@@ -450,12 +450,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * splits, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
       else tiled_gradx_kernel<W_E4M3, 2><<<4 * splits, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
     }
-    for (int hh = 0; hh < halves; hh++)
-      tiled_reduce_kernel<<<384, 64, 0, stream>>>(partial + (size_t)hh * part_half, splits, weight_type == W_BF16 ? 1 : 0, gx_total + (size_t)hh * BP * D);
-    const int ugrid = 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
+    const int ugrid = TRED_WAVES / 4 + 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
   tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, 256 * HV, (size_t)TUP_XBYTES * HV, stream>>>(                             \
-      w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0)
+      w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0, partial, part_half, splits,           \
+      weight_type == W_BF16 ? 1 : 0, gx_total)
 #define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                        \
   do {                                                                                                                         \
     if (halves == 1) XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 1, false); else XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 2, false);            \

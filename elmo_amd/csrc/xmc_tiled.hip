@@ -400,12 +400,15 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
   }
 }
 
-// sum of the partials of one chunk in a fixed order; bf16 weights: the chunk's contribution is rounded to bf16 before it
-// is added to the fp32 total (chunked.py:116)
-__global__ __launch_bounds__(64) void tiled_reduce_kernel(const floatx4* partial, int splits, int round_bf16, float* gx_total) {
-  // 384 workgroups of one wavefront: (slot, fb, wavefront of the grad_X kernel's layout); eight loads in flight
-  const int slot = blockIdx.x >> 4, fb = (blockIdx.x >> 2) & 3, wv = blockIdx.x & 3;
-  const int lane = threadIdx.x, tid = wv * 64 + lane, l16 = lane & 15, kg = lane >> 4;
+// sum of the partials of one chunk and batch half in a fixed order; bf16 weights: the chunk's contribution is rounded to
+// bf16 before it is added to the fp32 total (chunked.py:116).  Work of one wavefront; 384 of them cover a half.  It runs
+// in the first workgroups of the chunk's update launch (the two do not depend on each other), so the sum costs no
+// launch of its own and hides behind the update.
+constexpr int TRED_WAVES = 384;
+__device__ __forceinline__ void tiled_reduce_wave(int widx, int lane, const floatx4* partial, int splits, int round_bf16, float* gx_total) {
+  // (slot, fb, wavefront of the grad_X kernel's layout); eight loads in flight
+  const int slot = widx >> 4, fb = (widx >> 2) & 3, wv = widx & 3;
+  const int tid = wv * 64 + lane, l16 = lane & 15, kg = lane >> 4;
   floatx4 s = {0.f, 0.f, 0.f, 0.f};
   int sp = 0;
   for (; sp + 8 <= splits; sp += 8) {
@@ -531,13 +534,22 @@ constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of 
 template <int WT, int MODE, int HALVES, bool KAHAN>
 __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_update_kernel(
     void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, unsigned seed,
-    int saturate, void* kahan, int kahan_type, int num_head, unsigned label0) {
+    int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
+    int red_splits, int red_round_bf16, float* red_total) {
   static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
+  // the first workgroups sum the chunk's grad_X partials (384 wavefronts per batch half), the others update the weights
+  constexpr int RED_BLOCKS = TRED_WAVES * HALVES / (4 * HALVES);
+  if ((int)blockIdx.x < RED_BLOCKS) {
+    const int widx = (int)blockIdx.x * (4 * HALVES) + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
+    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_splits, red_round_bf16,
+                      red_total + (size_t)hh * BP * D);
+    return;
+  }
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = (tid >> 6) & 3, sub = tid >> 8, nsub = (int)blockDim.x >> 8;
   const int lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fb = blockIdx.x & 3, group = blockIdx.x >> 2;
+  const int fb = ((int)blockIdx.x - RED_BLOCKS) & 3, group = ((int)blockIdx.x - RED_BLOCKS) >> 2;
   // The X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and serves all tiles and
   // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
 #pragma unroll
