@@ -410,9 +410,8 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (n_pad > 0)
     quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys, nullptr);
   tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
-  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT);
-  tiled_zero_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>(gx_total, halves * BP * D);
-  if (loss_out) tiled_zero_kernel<<<(2 * num_tiles + 255) / 256, 256, 0, stream>>>(loss_part, 2 * num_tiles);
+  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT,
+                                                                        gx_total, loss_part, loss_out ? 2 * num_tiles : 0);
   for (int c = 0; c < num_chunks; c++) {
     void* w = chunk_ptrs[c];
     const int rows = c == num_chunks - 1 ? rows_last_chunk : rows_per_chunk;

@@ -50,9 +50,13 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 //       ones of chunked_fp8xmc_clf.py:101-102): block (nb, ks) = batch rows 16nb.. x features 32ks..
 //   xT: X^T for grad_W (never quantised): block (fblk, ks) = 16 features x batch rows 32ks.., the features of a block
 //       chosen so that a lane of the update kernel owns consecutive ones
-__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT) {
+// (also clears the fp32 grad_X total, one entry per thread, and the loss shares if there are any: no launches for that)
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT,
+                                    float* gx_total, float* loss_part, int n_loss) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
+  gx_total[i] = 0.f;
+  for (int j = i; j < n_loss; j += halves * BP * D) loss_part[j] = 0.f;
   int b = i / D, k = i - b * D;
   unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
   unsigned short vq = v;
