@@ -36,6 +36,8 @@ def load():
                                  ctypes.POINTER(ctypes.c_uint32), i32, f32, f32, vp, vp, vp, sz, vp]
     lib.xmc_fp8_forward.restype = i32
     lib.xmc_fp8_forward.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp, sz, vp]
+    lib.xmc_fp8_forward_static.restype = i32
+    lib.xmc_fp8_forward_static.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp]
     lib.xmc_step_error_word.restype = i32
     lib.xmc_step_error_word.argtypes = [vp, i32, i32, vp]
     lib.xmc_tiled_workspace_bytes.restype = sz

@@ -9,19 +9,32 @@
 
 using namespace xmc;
 
+// Operand images of X for xmc_fp8_forward_static, the entry point that takes no workspace: e4m3 X in MFMA operand order
+// (BP*D bytes), then the bf16 image the same preparation kernel writes (BP*D*2 bytes).  Every GPU the library runs on
+// holds its own copy of this array until the process ends.  In host code the name stands for the symbol only, never for
+// device memory: the address kernels get is the one hipGetSymbolAddress returned for the current device.
+constexpr size_t FWD_STATIC_XQ = 0;
+constexpr size_t FWD_STATIC_XT = (size_t)BP * D;
+constexpr size_t FWD_STATIC_BYTES = FWD_STATIC_XT + (size_t)BP * D * 2;   // 294,912
+static __device__ __align__(256) unsigned char scratch[FWD_STATIC_BYTES];
+
 namespace {
 
-struct DeviceInfo { int ok; int cus; };
+struct DeviceInfo { int ok; int cus; unsigned char* scratch_ptr; };
 
 DeviceInfo device_info() {
   static DeviceInfo cached[64] = {};
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DeviceInfo{-1, 0};
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DeviceInfo{-1, 0, nullptr};
   if (cached[dev].ok == 0) {
     hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DeviceInfo{-1, 0};
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DeviceInfo{-1, 0, nullptr};
     cached[dev].cus = prop.multiProcessorCount;
     cached[dev].ok = (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : -1;
+    // this device's copy of the static scratch array (device `dev` is current here); stays null if the lookup fails
+    void* sp = nullptr;
+    cached[dev].scratch_ptr = (cached[dev].ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess)
+                                  ? (unsigned char*)sp : nullptr;
     // opt in to the full 160 KiB of LDS once per device
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -94,6 +107,36 @@ int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_
 int topk_group(int rows_per_chunk) { const int g = (1 << 17) / rows_per_chunk; return g < 1 ? 1 : g; }
 size_t topk_zbuf_bytes(int rows_per_chunk) {
   return ((size_t)BP * topk_group(rows_per_chunk) * rows_per_chunk * 2 + 255) / 256 * 256;
+}
+
+// The launches of the inference logits, shared by xmc_fp8_forward (operand images in the caller's workspace) and
+// xmc_fp8_forward_static (operand images in this device's copy of the static array); shapes are checked by the callers.
+int forward_launch(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch, float scale_w,
+                   float scale_x, void* out_bf16, long long out_stride, long long num_labels, unsigned char* xq,
+                   unsigned short* xt, hipStream_t stream) {
+  if (!out_bf16) return XMC_ERR_NULL;
+  if (num_labels <= 0 || out_stride < num_labels || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
+  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, xq, xt);
+  ForwardParams fp;
+  for (int c = 0; c < MAX_CHUNKS; c++) fp.chunk[c] = c < num_chunks ? (const unsigned char*)chunk_ptrs[c] : nullptr;
+  fp.rows_per_chunk = rows_per_chunk;
+  fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
+  const int last_chunk = (int)((num_labels - 1) / rows_per_chunk);
+  fp.tile_begin = 0;
+  fp.tile_end = last_chunk * fp.tiles_per_chunk + (int)((num_labels - (long long)last_chunk * rows_per_chunk + FT - 1) / FT);
+  fp.xq = xq;
+  fp.zscale = scale_w * scale_x;
+  fp.out = (unsigned short*)out_bf16;
+  fp.out_stride = out_stride;
+  fp.col0 = 0;
+  fp.num_labels = num_labels;
+  fp.batch = batch;
+  const int grid = fp.tile_end < 2 * di.cus ? fp.tile_end : 2 * di.cus;   // two workgroups fit the LDS of a compute unit
+  fp8_forward_kernel<<<grid, NT, FWD_LDS, stream>>>(fp);
+  return launch_status();
 }
 
 }  // namespace
@@ -238,32 +281,31 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream_) {
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
-  if (!out_bf16) return XMC_ERR_NULL;
-  if (num_labels <= 0 || out_stride < num_labels || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
-  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
-  DeviceInfo di = device_info();
-  if (di.ok != 1) return XMC_ERR_DEVICE;
-  hipStream_t stream = (hipStream_t)stream_;
   unsigned char* ws = (unsigned char*)workspace;
-  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
-                                                              (unsigned short*)(ws + WS_XT));
-  ForwardParams fp;
-  for (int c = 0; c < MAX_CHUNKS; c++) fp.chunk[c] = c < num_chunks ? (const unsigned char*)chunk_ptrs[c] : nullptr;
-  fp.rows_per_chunk = rows_per_chunk;
-  fp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
-  const int last_chunk = (int)((num_labels - 1) / rows_per_chunk);
-  fp.tile_begin = 0;
-  fp.tile_end = last_chunk * fp.tiles_per_chunk + (int)((num_labels - (long long)last_chunk * rows_per_chunk + FT - 1) / FT);
-  fp.xq = ws + WS_XQ;
-  fp.zscale = scale_w * scale_x;
-  fp.out = (unsigned short*)out_bf16;
-  fp.out_stride = out_stride;
-  fp.col0 = 0;
-  fp.num_labels = num_labels;
-  fp.batch = batch;
-  const int grid = fp.tile_end < 2 * di.cus ? fp.tile_end : 2 * di.cus;   // two workgroups fit the LDS of a compute unit
-  fp8_forward_kernel<<<grid, NT, FWD_LDS, stream>>>(fp);
-  return launch_status();
+  return forward_launch(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, scale_w, scale_x, out_bf16, out_stride,
+                        num_labels, ws + WS_XQ, (unsigned short*)(ws + WS_XT), (hipStream_t)stream_);
+}
+
+int xmc_fp8_forward_static(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                           int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
+                           long long num_labels, void* stream_) {
+  // the same checks as xmc_fp8_forward, without a workspace; the static array holds the operand images of at most
+  // BP = 128 batch rows of D = 768 features, which is also the limit of xmc_fp8_forward
+  if (!chunk_ptrs || !x_bf16) return XMC_ERR_NULL;
+  if (features != D || batch <= 0 || batch > BP || batch % 16 != 0) return XMC_ERR_SHAPE;
+  if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return XMC_ERR_SHAPE;
+  if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
+  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1) return XMC_ERR_RANGE;
+  for (int c = 0; c < num_chunks; c++) {
+    if (!chunk_ptrs[c]) return XMC_ERR_NULL;
+    if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
+  }
+  if (!aligned16(x_bf16)) return XMC_ERR_ALIGN;
+  const DeviceInfo di = device_info();
+  if (di.ok != 1 || !di.scratch_ptr) return XMC_ERR_DEVICE;
+  return forward_launch(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, scale_w, scale_x, out_bf16, out_stride,
+                        num_labels, di.scratch_ptr + FWD_STATIC_XQ, (unsigned short*)(di.scratch_ptr + FWD_STATIC_XT),
+                        (hipStream_t)stream_);
 }
 
 size_t xmc_topk_scratch_bytes(int rows_per_chunk) {

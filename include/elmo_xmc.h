@@ -85,6 +85,17 @@ int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
                     long long num_labels, void* workspace, size_t workspace_bytes, void* stream);
 
+/* xmc_fp8_forward without a workspace argument.  It has no counterpart in the reference: it is for callers that cannot
+ * allocate device memory for a workspace (code under HIP graph capture, serving loops and harnesses that forbid
+ * hipMalloc).  The operand images of X that xmc_fp8_forward keeps in the caller's workspace live in a static device array
+ * of the library instead (294,912 bytes per GPU, held until the process ends), so the limits are those of the array:
+ * features == 768 and batch <= 128 (a multiple of 16); anything larger returns XMC_ERR_SHAPE.  The call allocates and
+ * frees nothing.  Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (two streams, two
+ * threads) race on it and must be serialised by the caller.  Outputs are bit-identical to xmc_fp8_forward's. */
+int xmc_fp8_forward_static(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                           int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
+                           long long num_labels, void* stream);
+
 /* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one group of chunks (up to 2^17 labels, or one
  * chunk of up to 2^18 rows) and the running lists (two of 128 entries per batch row). */
 size_t xmc_topk_scratch_bytes(int rows_per_chunk);
