@@ -315,7 +315,7 @@ def main():
     algo_flops = 6.0 * cfg.batch * cfg.num_labels * cfg.dim
     t_roof = max(algo_flops / (FP8_PEAK_TFLOPS * 1e12), algo_bytes / (HBM_PEAK_GBS * 1e9))
     achieved_gbs = algo_bytes / (kernel_ms * 1e-3) / 1e9
-    kernel_name = "fp8_step_kernel" if os.environ.get("XMC_KERNEL") == "pair" else "fp8_step_quad_kernel"
+    kernel_name = "fp8_step_quad_kernel"
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):

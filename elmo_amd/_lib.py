@@ -24,6 +24,20 @@ def load():
             f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
             "(hipcc --offload-arch=gfx950); there is no CPU fallback for the classifier step")
     lib = ctypes.CDLL(LIB_PATH)
+    # a library that predates an edit of the sources would run the old kernels: it reports the digest of the sources it
+    # was compiled from; on a mismatch it is rebuilt once, and if that is not possible the load fails
+    lib.xmc_source_hash.restype = ctypes.c_char_p
+    from . import build as _build
+    if LIB_PATH == _build.OUT and lib.xmc_source_hash().decode() != _build.source_hash():
+        del lib
+        try:
+            _build.build()
+        except Exception as e:
+            raise XmcError(f"{LIB_PATH} was built from other sources than those in the tree and could not be rebuilt: {e}")
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.xmc_source_hash.restype = ctypes.c_char_p
+        if lib.xmc_source_hash().decode() != _build.source_hash():
+            raise XmcError(f"{LIB_PATH} does not match the sources in the tree even after a rebuild")
     vp, i32, f32, sz, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_longlong
     lib.xmc_version.restype = i32
     lib.xmc_source_hash.restype = ctypes.c_char_p
@@ -50,8 +64,12 @@ def load():
     lib.xmc_fp8_forward_topk.restype = i32
     lib.xmc_fp8_forward_topk.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp, vp,
                                          vp, sz, vp, sz, vp]
-    lib.xmc_select_step_kernel.restype = i32
-    lib.xmc_select_step_kernel.argtypes = [i32]
+    lib.xmc_step_error_offset.restype = sz
+    lib.xmc_step_workgroups.restype = i32
+    lib.xmc_step_xcc_ids.restype = i32
+    lib.xmc_step_xcc_ids.argtypes = [vp, ctypes.POINTER(ctypes.c_int32), i32, vp]
+    lib.xmc_quad_placement_check.restype = i32
+    lib.xmc_quad_placement_check.argtypes = [ctypes.POINTER(ctypes.c_int32), i32]
     lib.xmc_copy_probe.restype = i32
     lib.xmc_copy_probe.argtypes = [vp, vp, sz, vp]
     lib.xmc_profile_events.restype = i32

@@ -1,7 +1,7 @@
 // extern "C" surface of libelmo_xmc.so: argument validation, workspace carving and kernel launches.
 // Declarations and the reference interfaces they replace: include/elmo_xmc.h.
 #include "../../include/elmo_xmc.h"
-#include "xmc_fp8_step.hip"
+#include "xmc_fp8_forward.hip"
 #include "xmc_fp8_quad.hip"
 #include "xmc_tiled.hip"
 #include "xmc_topk.hip"
@@ -36,9 +36,6 @@ DeviceInfo device_info() {
     cached[dev].scratch_ptr = (cached[dev].ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess)
                                   ? (unsigned char*)sp : nullptr;
     // opt in to the full 160 KiB of LDS once per device
-    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
@@ -64,8 +61,8 @@ DeviceInfo device_info() {
   return cached[dev];
 }
 
-// optional event pair recorded around the next launch of the fused step kernel (benchmarking aid)
-hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
+// optional event pair recorded around the next launch of the fused step kernel by the calling thread (benchmarking aid)
+thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
 
 inline bool aligned16(const void* q) { return ((uintptr_t)q & 15) == 0; }
 
@@ -88,16 +85,6 @@ int check_common(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
 // plain 16-byte-per-lane copy: the known-size reference against which memory counters are calibrated
 __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
-}
-
-// which fused kernel xmc_fp8_step launches: 0 = quad (default), 1 = pair; initial value from XMC_KERNEL=pair|quad
-int g_step_kernel = -1;
-int step_kernel_choice() {
-  if (g_step_kernel < 0) {
-    const char* e = getenv("XMC_KERNEL");
-    g_step_kernel = (e && !__builtin_strcmp(e, "pair")) ? 1 : 0;
-  }
-  return g_step_kernel;
 }
 
 int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
@@ -188,51 +175,13 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   hipStream_t stream = (hipStream_t)stream_;
   unsigned char* ws = (unsigned char*)workspace;
 
-  const int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;   // one workgroup per CU, pairs on one XCD
+  const int grid = di.cus < MAX_WG ? di.cus : MAX_WG;   // one workgroup per compute unit
   const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
   const int num_tiles = num_chunks * tiles_per_chunk;
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
-  if (step_kernel_choice() == 1) {
-    // a fill kernel, not a memset node: the step may be recorded into a graph by the caller
-    tiled_zero_kernel<<<4, 256, 0, stream>>>((float*)(ws + WS_FLAGS), 1024);
-    if (n_pad > 0)
-      quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch,
-                                                                            (unsigned*)(ws + WS_KEYS), nullptr);
-    tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>((const unsigned*)(ws + WS_KEYS), n_pad, rows_per_chunk,
-                                                                  tiles_per_chunk, num_tiles, (int*)(ws + WS_TILEPTR));
-    prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
-                                                                (unsigned short*)(ws + WS_XT));
-    StepParams p;
-    for (int c = 0; c < MAX_CHUNKS; c++) {
-      p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
-      p.seed[c] = (c < num_chunks && seeds) ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c]) : seeds[c]) : 0u;
-    }
-    p.num_chunks = num_chunks;
-    p.rows_per_chunk = rows_per_chunk;
-    p.tiles_per_chunk = tiles_per_chunk;
-    p.num_tiles = num_tiles;
-    p.xq = ws + WS_XQ;
-    p.xt = (const bf16x8*)(ws + WS_XT);
-    p.keys = (const unsigned*)(ws + WS_KEYS);
-    p.tile_ptr = (const int*)(ws + WS_TILEPTR);
-    p.partial = (floatx4*)(ws + WS_PARTIAL);
-    p.flags = (int*)(ws + WS_FLAGS);
-    p.zscale = scale_w * scale_x;
-    p.lr_eff = lr / scale_w;
-    p.batch = batch;
-    if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
-    switch (round_mode) {
-      case XMC_ROUND_RTN: fp8_step_kernel<ROUND_RTN><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-      case XMC_ROUND_SR_PHILOX: fp8_step_kernel<ROUND_SR_PHILOX><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-      default: fp8_step_kernel<ROUND_SR_FAST><<<grid, NT, LDS_BYTES, stream>>>(p); break;
-    }
-    if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
-    g_prof_start = g_prof_stop = nullptr;
-    reduce_gx_kernel<<<96, NT, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), grid, scale_w, grad_x_f32,
-                                           (unsigned short*)grad_x_bf16, batch);
-  } else {
+  {
     QuadParams p;
     for (int c = 0; c < MAX_CHUNKS; c++) {
       p.chunk[c] = c < num_chunks ? (unsigned char*)chunk_ptrs[c] : nullptr;
@@ -271,7 +220,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
     reduce_gx_quad_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
-                                                 (unsigned short*)grad_x_bf16, batch);
+                                                 (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
   }
   return launch_status();
 }
@@ -526,12 +475,6 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   return launch_status();
 }
 
-int xmc_select_step_kernel(int which) {
-  if (which < 0 || which > 1) return XMC_ERR_MODE;
-  g_step_kernel = which;
-  return XMC_OK;
-}
-
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream_) {
   if (!dst || !src) return XMC_ERR_NULL;
   if (!aligned16(dst) || !aligned16(src) || bytes % 16 != 0) return XMC_ERR_ALIGN;
@@ -543,15 +486,36 @@ int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream_) {
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream_) {
   (void)num_chunks; (void)rows_per_chunk;
   if (!workspace) return XMC_ERR_NULL;
-  DeviceInfo di = device_info();
-  if (di.ok != 1) return XMC_ERR_DEVICE;
-  int grid = (di.cus < MAX_WG ? di.cus : MAX_WG) / 16 * 16;
-  if (step_kernel_choice() == 0) grid = grid / 32 * 32;   // the quad kernel keeps the word behind its counters
   int word = 0;
-  if (hipMemcpyAsync(&word, (const unsigned char*)workspace + WS_FLAGS + (size_t)grid * 4, 4, hipMemcpyDeviceToHost,
+  if (hipMemcpyAsync(&word, (const unsigned char*)workspace + xmc_step_error_offset(), 4, hipMemcpyDeviceToHost,
                      (hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
   if (hipStreamSynchronize((hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
   return word;
+}
+
+size_t xmc_step_error_offset(void) { return WS_FLAGS + (size_t)QF_ERR * 4; }
+
+int xmc_step_workgroups(void) {
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  return (di.cus < MAX_WG ? di.cus : MAX_WG) / 32 * 32;
+}
+
+int xmc_step_xcc_ids(const void* workspace, int32_t* ids_host, int count, void* stream_) {
+  if (!workspace || !ids_host) return XMC_ERR_NULL;
+  if (count <= 0 || count > MAX_WG) return XMC_ERR_RANGE;
+  if (hipMemcpyAsync(ids_host, (const unsigned char*)workspace + WS_FLAGS + (size_t)QF_XCC * 4, (size_t)count * 4,
+                     hipMemcpyDeviceToHost, (hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream_) != hipSuccess) return XMC_ERR_LAUNCH;
+  return XMC_OK;
+}
+
+int xmc_quad_placement_check(const int32_t* xcc_ids_host, int num_workgroups) {
+  if (!xcc_ids_host) return XMC_ERR_NULL;
+  if (num_workgroups < 32 || num_workgroups > MAX_WG || num_workgroups % 32 != 0) return XMC_ERR_RANGE;
+  int bad = 0;
+  for (int q = 0; q < num_workgroups / 4; q++) bad += quad_xcc_mismatch(xcc_ids_host, q) ? 1 : 0;
+  return bad;
 }
 
 }  // extern "C"

@@ -14,31 +14,42 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-// ---- geometry (one MI355X compute unit works on a 64-label tile; a pair of CUs shares a tile, each
-//      owning one half of the 768 input features for the two gradient GEMMs and the update)
+// ---- geometry of the FP8 kernels
 constexpr int D = 768;            // input features (row length of W, bytes per FP8 row)
 constexpr int BP = 128;           // padded batch rows
-constexpr int TL = 64;            // labels per tile
-constexpr int NT = 256;           // threads per workgroup (4 wavefronts of 64)
-constexpr int HALF = D / 2;       // features owned by one CU of a pair
-constexpr int WCOLS = HALF / 4;   // features owned by one wavefront (96)
-constexpr int WS = D + 16;        // LDS row stride of the W tile, bytes (49 x 16)
-constexpr int GT_S = TL * 2 + 16; // LDS row stride of G^T [b][l], bytes
-constexpr int GL_S = BP * 2 + 16; // LDS row stride of G   [l][b], bytes
-constexpr int WT_BYTES = TL * WS;
-constexpr int LDS_BYTES = 2 * WT_BYTES + BP * GT_S + TL * GL_S;
+constexpr int TL = 64;            // labels per tile of the training kernels
+constexpr int NT = 256;           // threads per workgroup of the inference kernel (4 wavefronts of 64)
+constexpr int WS = D + 16;        // LDS row stride of a W tile in the inference kernel, bytes (49 x 16)
 constexpr int MAX_CHUNKS = 64;
 constexpr int MAX_POS = 16384;    // positives per step the single-workgroup sort handles
 
-// workspace layout (byte offsets), all 256-byte aligned
+// workspace of the fused step (byte offsets), all 256-byte aligned
 constexpr int MAX_WG = 256;                                   // workgroups of the persistent step kernel
 constexpr size_t WS_XQ = 0;                                   // FP8 logits operands   BP*D
 constexpr size_t WS_XT = WS_XQ + (size_t)BP * D;              // bf16 grad_W operands  BP*D*2
 constexpr size_t WS_KEYS = WS_XT + (size_t)BP * D * 2;        // sorted positive keys  MAX_POS*4
-constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // counters + error word (4 KiB), then 12 KiB of debug time stamps
-constexpr size_t WS_PARTIAL = WS_FLAGS + 16384;               // MAX_WG * 48 * 256 * 16 bytes of grad_X partials
-constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 48 * NT * 16;      // G exchange ring: 64 quads x 8 slots x 4 x 5 KiB
-constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 8 * 4 * 5120;  // tile_ptr[num_tiles + 1]
+constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // 1024 ints: counters, XCC ids, error word (below)
+constexpr size_t WS_PARTIAL = WS_FLAGS + 4096;                // MAX_WG * 12 * 512 * 16 bytes of grad_X partials
+constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 12 * 512 * 16;     // G exchange ring: 64 quads x 8 slots x 20 KiB
+constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 8 * 20480;   // tile_ptr[num_tiles + 1], then the tile descriptors
+
+// Layout of the 1024 ints at WS_FLAGS (cleared at the start of every step):
+//   [0, 256)              tiles-published / tiles-loaded counters of the persistent step kernels
+//   [QF_XCC, QF_XCC+256)  XCC id every workgroup of the quad kernel found itself on
+//   [QF_ERR]              error word: bit 0 = a bounded wait expired, bit 1 = the workgroups of a quad were not placed on
+//                         one XCD (their exchange of G through that XCD's L2 is then not coherent)
+constexpr int QF_XCC = 512;
+constexpr int QF_ERR = 1020;
+
+// The quad kernel assumes that workgroup g runs on XCD g % 8, and builds quads of four workgroups with equal g % 8:
+// member m of quad q is workgroup ((q / 8) * 4 + m) * 8 + q % 8.
+__host__ __device__ inline int quad_member_workgroup(int quad, int m) { return (((quad >> 3) << 2) + m) * 8 + (quad & 7); }
+// true if the four members of `quad` did not all record the same XCC id
+__host__ __device__ inline bool quad_xcc_mismatch(const int* xcc_ids, int quad) {
+  const int id0 = xcc_ids[quad_member_workgroup(quad, 0)];
+  return xcc_ids[quad_member_workgroup(quad, 1)] != id0 || xcc_ids[quad_member_workgroup(quad, 2)] != id0 ||
+         xcc_ids[quad_member_workgroup(quad, 3)] != id0;
+}
 
 __device__ __forceinline__ float bf16_rt(float f) { return (float)(__bf16)f; }
 

@@ -43,10 +43,7 @@ constexpr int QCOLS = D / 4;              // features owned by one member (192)
 constexpr int QWS = QCOLS + 16;           // LDS row stride of the own-column tile image (13 x 16 bytes)
 constexpr int QWC_BYTES = TL * QWS;       // 13312
 constexpr int QRING = 6;                  // own-column tile images: in use, four landed or landing, one in flight
-#ifndef XMC_GPAD
-#define XMC_GPAD 16
-#endif
-constexpr int QPL_S = TL * 2 + XMC_GPAD;  // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
+constexpr int QPL_S = TL * 2 + 16;        // bytes per batch row of the G tile ([128 b][64 l] bf16 + pad)
 constexpr int QG_PIECES = (BP * QPL_S + 1023) / 1024;   // wave-wide loads per G tile (18)
 constexpr int QG_BYTES = 20480;           // one G tile (128 x 144 = 18432), padded
 constexpr int QSLOTS = 8;                 // exchange slots per quad
@@ -57,7 +54,7 @@ constexpr int QROW_BYTES = 13 * 1024;     // 16 rows x 784 = 12544, padded to 13
 constexpr int QRRING = 3;                 // own-rows images in flight
 constexpr int QGBUF = 2;                  // gathered-G buffers: in use, in flight
 constexpr int QLDS_R = QLDS_G + QGBUF * QG_BYTES;
-constexpr int QLDS_M = QLDS_R + QRRING * QROW_BYTES;   // four snapshots of the counters, 16 bytes each
+constexpr int QLDS_M = QLDS_R + QRRING * QROW_BYTES;   // two snapshots of the counters, 16 bytes each; at +64 the abort word
 constexpr int QLDS_BYTES = QLDS_M + 256;
 constexpr int QSPIN_LIMIT = 1 << 18;
 constexpr int QAHEAD = 5;                 // stage A runs this many tiles ahead of stage B
@@ -77,19 +74,12 @@ struct QuadParams {
   const uint4* desc;                  // [num_tiles][2] tile descriptors written by quad_desc_prep_kernel
   floatx4* partial;                   // [gridDim.x][12][512] per-workgroup grad_X partial sums
   unsigned char* exch;                // [nquads][QSLOTS][QG_BYTES] G exchange ring
-  int* flags;                         // [nquads][4] tiles-published counters; [nquads*4] error word; then xcc ids
+  int* flags;                         // [nquads][4] tiles-published counters; [QF_XCC + g] XCC ids; [QF_ERR] error word
   float zscale;                       // scale_w * scale_x applied to the logits accumulator
   float lr_eff;                       // lr / scale_w
   int batch;
 };
 
-#ifdef XMC_TIMING   // timing experiments only: per-wavefront clock totals of the phases of the main loop
-#define QT_DECL unsigned long long tprev = __builtin_amdgcn_s_memtime(); unsigned tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#define QT(k) { __builtin_amdgcn_sched_barrier(0); unsigned long long tn = __builtin_amdgcn_s_memtime(); tacc[k] += (unsigned)(tn - tprev); tprev = tn; __builtin_amdgcn_sched_barrier(0); }
-#else
-#define QT_DECL
-#define QT(k)
-#endif
 #define QFENCE() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point
 typedef __attribute__((address_space(3))) unsigned char qlds_u8;
 typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -294,8 +284,11 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
   // the sorted keys are written before this kernel starts: read them through the scalar (constant) path
   const __attribute__((address_space(4))) unsigned* ckeys = (const __attribute__((address_space(4))) unsigned*)p.keys;
   int* flags = p.flags + quad * 4;
-  int* errw = p.flags + nquads * 4;
-  if (tid == 0) p.flags[nquads * 4 + 1 + g] = (int)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15);   // XCC_ID
+  int* errw = p.flags + QF_ERR;
+  // the XCD this workgroup really runs on: reduce_gx_quad_kernel compares the four members of every quad
+  if (tid == 0) p.flags[QF_XCC + g] = (int)(__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15);   // XCC_ID
+  // abort word of the workgroup: set by a wavefront whose bounded wait expired, read by all after the next barrier
+  if (tid == 0) *(__attribute__((address_space(3))) int*)(lds + QLDS_M + 64) = 0;
 
   // ---- resident operands
   intx8 xq[6];         // logits: batch block 16v.., K steps of 128
@@ -312,7 +305,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 #pragma unroll
     for (int b = 0; b < 3; b++) acc2[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  QT_DECL
   // Per-lane source rows and byte offsets of the wave-wide pieces this wavefront loads (pieces v and v+8 of an image).
   // own-column image: 64 rows x 13 chunks of 16 bytes (12 data + 1 pad) = 13 pieces of 1 KiB
   // own-rows image:   rows 16m..16m+15, 16 x 50 chunks of 16 bytes (48 data + 2 pad) = 13 pieces
@@ -444,7 +436,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       int f = __hip_atomic_load(flags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (__builtin_amdgcn_read_exec() == __builtin_amdgcn_ballot_w64(f >= need)) break;
       if (spin >= QSPIN_LIMIT || ((spin & 1023) == 1023 && __hip_atomic_load(errw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-        if (lane == 0) __hip_atomic_store(errw, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // give up: raise the error word (partners that wait for this workgroup see it and give up too) and the
+        // workgroup's abort word; the iteration under way still has valid G, the next one is not started
+        if (lane == 0) {
+          __hip_atomic_fetch_or(errw, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          *(__attribute__((address_space(3))) int*)(lds + QLDS_M + 64) = 1;
+        }
         break;
       }
       __builtin_amdgcn_s_sleep(2);
@@ -507,9 +504,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     if (!prev_regular) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     else if (h == 0) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)" ::: "memory");
-    QT(0)
     __syncthreads();
-    QT(1)
+    // a wavefront gave up waiting in the iteration before: G of this position may be missing, nothing more is
+    // computed or stored (the weights of the remaining tiles stay as they were; the error word tells the host)
+    if (__builtin_amdgcn_readfirstlane(*(const __attribute__((address_space(3))) int*)(lds + QLDS_M + 64)) != 0) break;
     const QTile q = q_n, qa = qa_n, qr = qr_n, qw = qw_n;
     int fmin = fboot;
     if (i >= 1) {   // the counters as they were one iteration ago
@@ -536,13 +534,11 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       else if (k < 7) rows_piece(slot_rows, qr, k - 5);
     };
     mem_piece(0);
-    QT(2)
 
     // The two wavefronts of a SIMD run stage A and grad_X in opposite orders, so that the LDS reads of one overlap
     // the MFMAs of the other.
     if (h == 0 && do_a) stage_a(i + QAHEAD, slot_a, qa);
     mem_piece(1);
-    QT(3)
 
     // ---- grad_X[64 x 48] += G^T W; 6 steps (32-row K step major, 16-feature block minor); the transposed W read of
     //      step s+2 and the fp8->bf16 conversion of step s+1 are issued between the MFMAs of step s
@@ -573,7 +569,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
       }
     }
     if (h != 0 && do_a) stage_a(i + QAHEAD, slot_a, qa);
-    QT(4)
 
     qa_n = q_desc_full(cdesc, tile_at(i + 1 + QAHEAD));
     qr_n = q_desc_head(cdesc, tile_at(i + 1 + QAHEAD + 2));
@@ -657,16 +652,11 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         }
       }
     }
-    QT(5)
     { const int t = s0; s0 = s1; s1 = s2; s2 = t; }
     w0 = w0 == QRING - 1 ? 0 : w0 + 1;
   }
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last descriptor fetches still target LDS
-#ifdef XMC_TIMING
-  if (lane == 0 && g < 48)
-    for (int k = 0; k < 8; k++) p.flags[1024 + (g * 8 + v) * 8 + k] = (int)tacc[k];
-#endif
   // ---- per-workgroup grad_X partial, summed in a fixed order by reduce_gx_quad_kernel
   floatx4* dst = p.partial + (size_t)g * 12 * QNT;
 #pragma unroll
@@ -678,7 +668,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 // grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768].  192 workgroups of 128
 // threads: workgroup (slot, m, part) covers threads 128 part.. of the step kernel's workgroup layout.
 __global__ __launch_bounds__(128) void reduce_gx_quad_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
-                                                             unsigned short* gx_bf16, int batch) {
+                                                             unsigned short* gx_bf16, int batch, int* flags) {
+  // placement check: the members of a quad exchanged G through the L2 of one XCD, which holds only if all four ran there
+  if (blockIdx.x == 0 && (int)threadIdx.x < (nwg >> 2) && quad_xcc_mismatch(flags + QF_XCC, (int)threadIdx.x))
+    __hip_atomic_fetch_or(flags + QF_ERR, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const int slot = blockIdx.x >> 4, m = (blockIdx.x >> 2) & 3;   // slot = mb*3+nn
   const int tid = (blockIdx.x & 3) * 128 + threadIdx.x, v = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   const int fg = v & 3, h = v >> 2;

@@ -209,5 +209,10 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
     return (grad_out, gf) if want_f32 else grad_out
 
 
+def step_error_offset():
+    """Byte offset of the fused step's error word (int32) inside its workspace."""
+    return int(_lib.load().xmc_step_error_offset())
+
+
 def step_error_word(workspace, num_chunks, rows_per_chunk):
     return _lib.load().xmc_step_error_word(workspace.data_ptr(), num_chunks, rows_per_chunk, _stream_ptr())

@@ -81,6 +81,12 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
         self._tiled_workspace = None
         self._fused_ran = False      # the error word in the workspace is defined once a fused step has run
+        # After every fused step the error word is copied to pinned host memory on the step's stream, without waiting;
+        # the next step looks at copies that have arrived (see _check_previous_steps).
+        off = ops.step_error_offset()
+        self._err_dev = self._workspace[off:off + 4].view(torch.int32)
+        self._err_host = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self._err_event = None
         # batches of more than 128 rows (up to 256) also run on the three-kernel path, with the true-FP8 arithmetic
         self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
@@ -92,12 +98,23 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
     def _chunks(self):
         return [w.data for w in self.xfc_weight]
 
+    def _simulated_logits(self, embed):
+        # simulated FP8 (:51-52): matmul(embed.bf16, W.bf16) per chunk with the embedding as it comes - NOT quantised
+        # to e4m3, unlike the true-FP8 branch (:53-56).  (The evaluator casts the embedding to e4m3 itself before the
+        # call, evaluate.py:155-156; such an input is widened exactly.)  A library bf16 GEMM per chunk, as in the
+        # reference; this debugging mode has no kernel of its own here.
+        x = embed.to(torch.bfloat16)
+        outs = [torch.matmul(x, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
+        return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
+
     @torch.no_grad()
     def xfc_forward(self, embed):
         '''
         Mainly used during inference: logits [B, cfg.data.num_labels] in bf16 (padding rows dropped).
         '''
         assert embed.is_cuda and embed.dim() == 2
+        if self.fake_fp8_matmul:
+            return self._simulated_logits(embed)
         return ops.fp8_forward(self._chunks(), embed, self.cfg.data.num_labels, self.scale_w, self.scale_x,
                                self._workspace)
 
@@ -108,6 +125,9 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         [B, num_labels] logits: the top-k is merged chunk by chunk.  Not in the reference; k <= 128.
         '''
         assert embed.is_cuda and embed.dim() == 2
+        if self.fake_fp8_matmul:
+            vals, idx = self._simulated_logits(embed).topk(k)
+            return vals, idx
         return ops.fp8_forward_topk(self._chunks(), embed, self.cfg.data.num_labels, k, self.scale_w, self.scale_x,
                                     self._workspace)
 
@@ -156,11 +176,29 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
                                              round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
                                              saturate=True)
         else:
+            self._check_previous_steps()
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
                                            scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
             self._fused_ran = True
+            # the step's error word follows it on the stream into pinned host memory; nobody waits for it here
+            self._err_host.copy_(self._err_dev, non_blocking=True)
+            self._err_event = torch.cuda.Event()
+            self._err_event.record()
         self.iteration += 1
         return loss
+
+    def _check_previous_steps(self):
+        """Raises if a fused step whose error word has reached the host reported a failure (never waits: a word that is
+        still on its way is looked at by a later call)."""
+        if self._err_event is not None and self._err_event.query():
+            word = int(self._err_host[0])
+            if word != 0:
+                self._err_host[0] = 0
+                raise RuntimeError(
+                    f"fused classifier step failed (error word {word}): "
+                    + ("a workgroup gave up waiting for its partners (another stream kept the device busy?); " if word & 1 else "")
+                    + ("the workgroups of a quad were not placed on one XCD; " if word & 2 else "")
+                    + "the weights and grad_input of that step are incomplete")
 
     def last_step_error(self):
         """Error word of the last fused step (0 = fine; non-zero = a workgroup gave up waiting for its partners, e.g.

@@ -82,6 +82,11 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
         Mainly used during inference: logits [B, cfg.data.num_labels] in bf16 (padding rows dropped, :71).
         '''
         assert embed.is_cuda and embed.dim() == 2
+        if self.fake_fp8_matmul:
+            # simulated FP8 (:62-63): a bf16 GEMM per chunk on the embedding as it comes, not quantised to e4m3
+            x = embed.to(torch.bfloat16)
+            outs = [torch.matmul(x, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
+            return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
         return ops.fp8_forward(self._chunks(), embed, self.cfg.data.num_labels, 1.0, 1.0, self._workspace)
 
     @torch.no_grad()

@@ -68,8 +68,9 @@ size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk);
  * per compute unit, and the four workgroups that share a tile stream wait for one another through counters in the
  * workspace, so all of them must be running at the same time.  Give the step the whole device while it runs: a kernel
  * of another stream that keeps compute units occupied for more than about ten milliseconds makes the waiting
- * workgroups give up (every wait is bounded; nothing hangs) - the step's results are then invalid and the error word
- * (xmc_step_error_word) is non-zero.  One step at a time per workspace.
+ * workgroups give up (every wait is bounded; nothing hangs).  A workgroup that gives up stops before its next tile, so
+ * no weight is ever updated from missing data; the step is incomplete and the error word (xmc_step_error_word,
+ * xmc_step_error_offset) is non-zero.  One step at a time per workspace.
  */
 int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
                  int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
@@ -156,20 +157,31 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
                    int num_head, void* grad_x_bf16, float* grad_x_f32, float* loss_out, void* workspace,
                    size_t workspace_bytes, void* stream);
 
-/* Selects the fused kernel that xmc_fp8_step launches (no counterpart in the reference): 0 = four compute units per
- * tile stream without repeated arithmetic (default), 1 = two compute units per tile stream with the logits computed
- * twice.  Both produce the same weights; grad_X differs by fp32 summation order only.  The environment variable
- * XMC_KERNEL=pair|quad sets the initial choice. */
-int xmc_select_step_kernel(int which);
-
 /* Measurement aid (no counterpart in the reference): copies `bytes` (a multiple of 16) from src to dst with a plain
  * grid-stride kernel.  Memory-traffic counters are calibrated against this launch of known size. */
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
 
-/* Reads back the error word the last step on this workspace left there (non-zero: a workgroup gave up waiting for its
- * partner, see xmc_fp8_step; every step clears the word when it starts).  Synchronises the stream: meant for tests,
- * debugging and a check where the training loop synchronises anyway, not for every step. */
+/* Reads back the error word the last fused step on this workspace left there (every step clears it when it starts):
+ *   bit 0  a workgroup gave up waiting for its partners (see xmc_fp8_step); it and, in turn, its partners stopped at
+ *          that tile: the weights of the tiles they had not reached are unchanged, grad_X is incomplete
+ *   bit 1  the four workgroups of some quad did not run on one XCD (a partition mode or dispatch order the kernel
+ *          does not expect): the G they exchanged through that XCD's L2 may have been stale, the step is invalid
+ * Synchronises the stream: meant for tests, debugging and a check where the training loop synchronises anyway. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
+
+/* Byte offset of that error word (one int32) inside the workspace, for callers that want to copy it to pinned host
+ * memory asynchronously after every step instead of synchronising (the Python module does). */
+size_t xmc_step_error_offset(void);
+
+/* Diagnostics of the placement assumption of the fused kernel (no counterpart in the reference).  The kernel builds
+ * quads out of workgroups g with equal g % 8 and expects them on one XCD; every workgroup records the XCC id it really
+ * ran on.  xmc_step_workgroups: number of workgroups the fused kernel is launched with on the current device.
+ * xmc_step_xcc_ids: copies the ids of the first `count` workgroups of the last step to host memory (synchronises).
+ * xmc_quad_placement_check: host-only; number of quads whose four members recorded different ids (0 = fine) - the
+ * comparison the device makes at the end of every step before it raises bit 1 of the error word. */
+int xmc_step_workgroups(void);
+int xmc_step_xcc_ids(const void* workspace, int32_t* ids_host, int count, void* stream);
+int xmc_quad_placement_check(const int32_t* xcc_ids_host, int num_workgroups);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,7 @@ def test_every_declared_symbol_is_exported():
     lib = _lib.load()
     names = declared_functions()
     assert {"xmc_version", "xmc_error_string", "xmc_workspace_bytes", "xmc_fp8_step", "xmc_fp8_forward",
-            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_select_step_kernel", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes"} <= set(names)
+            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -47,8 +47,8 @@ def test_workspace_bytes():
     lib = _lib.load()
     a = lib.xmc_workspace_bytes(11, 60928)
     b = lib.xmc_workspace_bytes(2, 64)
-    assert a > b > 50 * 2 ** 20 and a % 256 == 0       # grad_X partials dominate: about 50 MiB
-    assert a < 80 * 2 ** 20
+    assert a > b > 34 * 2 ** 20 and a % 256 == 0       # grad_X partials (24 MiB) and the G exchange ring (10 MiB) dominate
+    assert a < 40 * 2 ** 20
     assert lib.xmc_workspace_bytes(0, 64) == 0 and lib.xmc_workspace_bytes(65, 64) == 0 and lib.xmc_workspace_bytes(2, 0) == 0
 
 
@@ -89,3 +89,33 @@ def test_python_wrapper_raises_on_error_status():
     with pytest.raises(_lib.XmcError):
         _lib.check(-2, "xmc_fp8_step")
     _lib.check(0, "xmc_fp8_step")
+
+
+def test_quad_placement_comparison():
+    """The comparison the device makes at the end of every fused step (the four workgroups of a quad must have recorded
+    one XCC id), on the host: the placement the kernel assumes passes, any member elsewhere is counted."""
+    lib = _lib.load()
+    n = 256
+    ids = (ctypes.c_int32 * n)(*[g % 8 for g in range(n)])             # workgroup g on XCD g % 8
+    assert lib.xmc_quad_placement_check(ids, n) == 0
+    ids[8 * 5 + 3] = 4                                                 # workgroup 43 = member 1 of quad 8*1+3 ran on XCD 4
+    assert lib.xmc_quad_placement_check(ids, n) == 1
+    ids2 = (ctypes.c_int32 * n)(*[(g // 4) % 8 for g in range(n)])     # four consecutive workgroups per XCD: every quad is split
+    assert lib.xmc_quad_placement_check(ids2, n) == n // 4
+    ids3 = (ctypes.c_int32 * n)(*[(g + 3) % 8 for g in range(n)])      # a rotated but consistent placement is fine
+    assert lib.xmc_quad_placement_check(ids3, n) == 0
+    assert lib.xmc_quad_placement_check(None, n) == -1
+    assert lib.xmc_quad_placement_check(ids, 40) == -4
+    assert lib.xmc_step_error_offset() % 4 == 0
+
+
+def test_static_forward_rejects_bad_arguments_before_touching_the_device():
+    lib = _lib.load()
+    P = 0x7F0000001000
+    arr = (ctypes.c_void_p * 1)(P)
+    call = lambda **k: lib.xmc_fp8_forward_static(k.get("arr", arr), k.get("nc", 1), k.get("rows", 64), k.get("x", P), k.get("batch", 16),
+                                                  k.get("feat", 768), 1.0, 1.0, P, 64, 64, None)
+    assert call(arr=None) == -1 and call(x=None) == -1
+    assert call(batch=144) == -2 and call(batch=8) == -2 and call(feat=1024) == -2 and call(rows=40) == -2
+    assert call(nc=65) == -4
+    assert call(x=P + 2) == -3

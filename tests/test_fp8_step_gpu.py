@@ -63,16 +63,29 @@ def test_rtn_parity_small(gpu, nc, rows, batch, seed):
     check_rtn(case, gpu)
 
 
-@pytest.mark.parametrize("nc,rows,batch,seed", [(3, 208, 32, 13), (5, 2000, 64, 15), (2, 4096, 128, 14)])
-def test_rtn_parity_pair_kernel(gpu, nc, rows, batch, seed):
-    """The alternative fused kernel (two compute units per tile stream) meets the same bar."""
-    from elmo_amd import _lib
+def test_quads_run_on_one_xcd_each(gpu):
+    """The four workgroups of a quad exchange G through the L2 of one XCD.  After a step the XCC ids the workgroups
+    recorded are read back: every quad's four are equal (the device makes the same comparison at the end of the step
+    and raises bit 1 of the error word otherwise), and the error word is clear."""
+    import ctypes
+    import torch
+    from elmo_amd import _lib, ops
     lib = _lib.load()
-    _lib.check(lib.xmc_select_step_kernel(1), "xmc_select_step_kernel")
-    try:
-        check_rtn(H.make_case(nc, rows, batch, seed), gpu)
-    finally:
-        _lib.check(lib.xmc_select_step_kernel(0), "xmc_select_step_kernel")
+    case = H.make_case(2, 4096, 32, 17)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    ws = ops.alloc_workspace(2, 4096, gpu)
+    ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws)
+    n = lib.xmc_step_workgroups()
+    assert n >= 32 and n % 32 == 0
+    ids = (ctypes.c_int32 * n)()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.xmc_step_xcc_ids(ws.data_ptr(), ids, n, stream), "xmc_step_xcc_ids")
+    assert lib.xmc_quad_placement_check(ids, n) == 0, list(ids)
+    assert len(set(ids)) == 8 and all(0 <= v < 8 for v in ids)      # eight XCDs, all in use
+    assert ops.step_error_word(ws, 2, 4096) == 0
+    # the asynchronous form of the error check (what the module does after every step)
+    off = lib.xmc_step_error_offset()
+    assert int(ws[off:off + 4].view(torch.int32).item()) == 0
 
 
 def test_rtn_parity_medium_full_batch(gpu):

@@ -131,3 +131,54 @@ def test_error_convention(gpu):
         build(gpu, 1000, 2, simulated=True, rounding="sr_fast")
     with pytest.raises(AssertionError):
         build(gpu, 1000, 2, simulated=True, scale_w=0.5)
+
+
+def test_simulated_mode_forward_uses_the_unquantised_embedding(gpu):
+    """chunked_fp8xmc_clf.py:51-52: in simulated-FP8 mode the inference logits are matmul(embed.bf16, W.bf16) - the
+    embedding is NOT quantised to e4m3 there (the true-FP8 branch :53-56 quantises it).  Checked against the closed form
+    on the CPU (exact products of bf16 x e4m3 values summed in float64, rounded to bf16) for a bf16 embedding, and
+    against the true-FP8 layer for an embedding the evaluator has already cast to e4m3 (evaluate.py:155-156)."""
+    import torch
+    xfc = build(gpu, 1000, 2, simulated=True)
+    xfc8 = build(gpu, 1000, 2)
+    for a, b in zip(xfc8.xfc_weight, xfc.xfc_weight):
+        a.data.copy_(b.data)
+    torch.manual_seed(4)
+    embed = torch.randn(24, 768, device=gpu).to(torch.bfloat16)
+    logits = xfc.xfc_forward(embed)
+    assert logits.shape == (24, 1000) and logits.dtype == torch.bfloat16
+    w = np.concatenate([C.e4m3_decode(p.view(torch.uint8).cpu().numpy()) for p in xfc.xfc_weight])[:1000]
+    x = embed.float().cpu().numpy()
+    exact = x.astype(np.float64) @ w.astype(np.float64).T
+    H.assert_bf16_close(logits.float().cpu().numpy(), C.bf16_round(exact.astype(np.float32)))
+    # the quantised product differs visibly: the two modes must not be confused
+    q = xfc8.xfc_forward(embed).float().cpu().numpy()
+    assert np.abs(q - exact).max() > 4 * np.abs(logits.float().cpu().numpy() - exact).max()
+    # an embedding that is already e4m3 gives the same logits in both modes, up to the summation order of the GEMM
+    e8 = embed.to(torch.float8_e4m3fn)
+    H.assert_bf16_close(xfc.xfc_forward(e8).float().cpu().numpy(), xfc8.xfc_forward(e8).float().cpu().numpy())
+    tv, ti = xfc.xfc_forward_topk(embed, 5)
+    assert torch.equal(tv, logits.topk(5).values) and torch.equal(logits.gather(1, ti), tv)
+
+
+def test_module_reports_a_failed_step_without_synchronising(gpu):
+    """After every fused step the module sends the step's error word to pinned host memory behind the step; the next
+    call raises if a word that has arrived is non-zero.  The failure is staged from the host (the word in the workspace is
+    overwritten before the copy is enqueued), every kernel runs normally."""
+    import torch
+    xfc = build(gpu, 1000, 2, rounding="rtn")
+    x = torch.randn(16, 768, device=gpu).to(torch.bfloat16)
+    labels = torch.zeros((0, 2), dtype=torch.int32, device=gpu)
+    xfc.xfc_forward_backward(x, labels, [0.05])
+    torch.cuda.synchronize()
+    xfc._check_previous_steps()                          # a clean step: nothing raised
+    assert int(xfc._err_host[0]) == 0
+    xfc._err_dev.fill_(2)                                # as if the placement check of that step had failed
+    xfc._err_host.copy_(xfc._err_dev, non_blocking=True)
+    xfc._err_event.record()
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="XCD"):
+        xfc.xfc_forward_backward(x, labels, [0.05])
+    xfc.xfc_forward_backward(x, labels, [0.05])          # reported once; the next step runs (and clears the word)
+    torch.cuda.synchronize()
+    assert xfc.last_step_error() == 0
