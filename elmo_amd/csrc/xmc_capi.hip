@@ -155,7 +155,8 @@ const char* xmc_error_string(int status) {
 size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk) {
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
   size_t tiles = (size_t)num_chunks * ((rows_per_chunk + TL - 1) / TL);
-  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256 + tiles * 32;   // tile_ptr, then 32-byte tile descriptors
+  // tile_ptr, then 32-byte tile descriptors, one run per quad (up to MAX_WG / 4 runs, each rounded up to whole entries)
+  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256 + (tiles + MAX_WG / 4) * 32;
 }
 
 int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
@@ -205,6 +206,8 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.batch = batch;
     const int qgrid = grid / 32 * 32;   // whole quads on every XCD
     if (qgrid < 32) return XMC_ERR_DEVICE;
+    p.nquads = qgrid >> 2;
+    p.kmax = (num_tiles + p.nquads - 1) / p.nquads;
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
         labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;

@@ -71,7 +71,10 @@ struct QuadParams {
   const bf16x8* xt;                   // grad_W operands
   const unsigned* keys;               // sorted positives: label*256 + batch_row
   const int* tile_ptr;                // [num_tiles+1] offsets into keys
-  const uint4* desc;                  // [num_tiles][2] tile descriptors written by quad_desc_prep_kernel
+  const uint4* desc;                  // [nquads][kmax][2] tile descriptors written by quad_desc_prep_kernel: the tiles of
+                                      // one quad are consecutive entries, in the order the quad walks them
+  int nquads;                         // quads of the step kernel's launch (grid / 4)
+  int kmax;                           // descriptor entries per quad = ceil(num_tiles / nquads)
   floatx4* partial;                   // [gridDim.x][12][512] per-workgroup grad_X partial sums
   unsigned char* exch;                // [nquads][QSLOTS][QG_BYTES] G exchange ring
   int* flags;                         // [nquads][4] tiles-published counters; [QF_XCC + g] XCC ids; [QF_ERR] error word
@@ -262,8 +265,11 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
     const int c = t / p.tiles_per_chunk;
     const int row0 = (t - c * p.tiles_per_chunk) * TL;
     const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
-    desc[2 * t] = uint4{(unsigned)base, (unsigned)(base >> 32), (unsigned)min(TL, p.rows_per_chunk - row0), p.seed[c]};
-    desc[2 * t + 1] = uint4{(unsigned)p0, (unsigned)p1, (unsigned)row0, (unsigned)(c * p.rows_per_chunk + row0)};
+    // tile t is position t / nquads of quad t % nquads: a quad reads its descriptors as one contiguous run, so the
+    // scalar cache serves all but one fetch in two
+    const int slot = (t % p.nquads) * p.kmax + t / p.nquads;
+    desc[2 * slot] = uint4{(unsigned)base, (unsigned)(base >> 32), (unsigned)min(TL, p.rows_per_chunk - row0), p.seed[c]};
+    desc[2 * slot + 1] = uint4{(unsigned)p0, (unsigned)p1, (unsigned)row0, (unsigned)(c * p.rows_per_chunk + row0)};
   }
 }
 
@@ -325,9 +331,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
     roff_full[s] = rows_offset(s, TL - 1);
   }
   q_cdesc* cdesc = (q_cdesc*)p.desc;
-  // tile index of position k in this quad's sequence; positions past the end fall back to tile 0, whose data is
-  // loaded and never used
-  auto tile_at = [&](int k) { const int t = quad + nquads * k; return t < p.num_tiles ? t : 0; };
+  // descriptor entry of position k in this quad's sequence; positions past the end fall back to entry 0 (tile 0),
+  // whose data is loaded and never used
+  auto tile_at = [&](int k) { return k < n_it ? quad * p.kmax + k : 0; };
   auto wcol_piece = [&](int slot, const QTile& q, int s) {
     if (v + 8 * s >= 13) return;
     if (q.rows_valid == TL) q_lds_load16_sbase(q.base, woff_full[s], (unsigned)(slot * QWC_BYTES + (v + 8 * s) * 1024));
