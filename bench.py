@@ -61,6 +61,34 @@ def cpu_baseline(cfg, budget_s=12.0):
     }
 
 
+def device_settle(lib, dev, want_ms):
+    """Keeps the device busy with the library's plain copy kernel and a library bf16 GEMM for about want_ms milliseconds
+    before the warm-up steps.  A device that has been idle runs its first ~20 ms of sustained work through a clock/power transient (the
+    same step kernel takes 0.48, then up to 0.59, then 0.46 ms over the first 40 launches of a process); the copy
+    kernel is not a step and touches none of the step's buffers.  Returns the milliseconds spent."""
+    import torch
+    if want_ms <= 0:
+        return 0.0
+    from elmo_amd import _lib
+    n = 256 << 20
+    src = torch.zeros(n, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    ga = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    gb = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < want_ms:
+        for _ in range(4):      # memory traffic and matrix-core work, as the step has both
+            _lib.check(lib.xmc_copy_probe(dst.data_ptr(), src.data_ptr(), n, stream), "xmc_copy_probe")
+            torch.matmul(ga, gb)
+        torch.cuda.synchronize()
+    spent = (time.perf_counter() - t0) * 1e3
+    del src, dst, ga, gb
+    torch.cuda.empty_cache()
+    return spent
+
+
 def bench_tiled(args, cfg):
     """The secondary modes (bf16 layer, simulated FP8, true FP8 with a batch above 128): three kernels per chunk and
     batch half; timed as a whole step with HIP events on the torch stream."""
@@ -215,6 +243,8 @@ def main():
     ap.add_argument("--round", default="sr_fast", choices=["sr_fast", "sr_philox", "rtn"])
     ap.add_argument("--mode", default="step", choices=["step", "forward", "forward_topk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="milliseconds of plain copy kernels before the warm-up steps (clock settling of an idle device); 0 = none")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only launch the library's plain copy kernel over MIB MiB five times (counter calibration) and exit")
     args = ap.parse_args()
@@ -292,6 +322,7 @@ def main():
         assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
         events.append((a, b))
 
+    settle_ms = device_settle(lib, dev, args.settle_ms)
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
@@ -371,11 +402,14 @@ def main():
                      "kernel": kernel_name,
                      "kernel_ms": kernel_ms,
                      "kernel_ms_stats": {"median": float(np.median(kms)), "p10": float(np.percentile(kms, 10)),
-                                         "p90": float(np.percentile(kms, 90)), "min": float(kms.min()), "max": float(kms.max())},
+                                         "p90": float(np.percentile(kms, 90)), "min": float(kms.min()), "max": float(kms.max()),
+                                         "first_8": [round(float(v), 4) for v in kms[:8]],
+                                         "last_8": [round(float(v), 4) for v in kms[-8:]]},
                      "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_flops_per_launch": algo_flops},
         "roofline_step_frac": t_roof / (ms_per_step * 1e-3),
         "roofline_steps_per_s": 1.0 / t_roof,
         "peak_hbm_gb": peak_bytes / 1e9, "peak_hbm_over_weights": peak_bytes / weight_bytes,
+        "device_settle_ms_before_warmup": settle_ms,
         "rounding_modes": modes,
         "rounding_note": "value is measured with config.rounding; sr_fast is this build's own unbiased stochastic rounding "
                          "(not the reference's random stream), sr_philox the reference's Philox bit recipe",
