@@ -260,14 +260,20 @@ def bf16_forward(w_bf16, x_bf16):
     return C.bf16_round(z)
 
 
-def scalar_fp8_step_tiny(w_codes, x_bf16, labels, lr, scale_w=1.0, scale_x=1.0):
+def scalar_fp8_step_tiny(w_codes, x_bf16, labels, lr, scale_w=1.0, scale_x=1.0, simulated=False):
     """Brute-force scalar loops (pure Python floats = float64) for tiny inputs; RTN mode, one chunk.
-    Independent of the vectorised code above except for the scalar codecs."""
+    Independent of the vectorised code above except for the scalar codecs.
+    simulated (chunked_fp8xmc_clf.py:98-99,110,115-116): the logits take X as it is (bf16, not quantised to e4m3) and
+    the final cast is torch's (no saturation: NaN above 464); everything else is the same arithmetic."""
     L, d = w_codes.shape
     B = x_bf16.shape[0]
     dec = [float(v) for v in C.E4M3_TABLE]
     w = [[dec[int(w_codes[l, k])] for k in range(d)] for l in range(L)]
-    xq = [[dec[int(C.e4m3_encode(np.float32(x_bf16[b, k]) / np.float32(scale_x)))] for k in range(d)] for b in range(B)]
+    if simulated:
+        assert scale_w == 1.0 and scale_x == 1.0
+        xq = [[float(x_bf16[b, k]) for k in range(d)] for b in range(B)]
+    else:
+        xq = [[dec[int(C.e4m3_encode(np.float32(x_bf16[b, k]) / np.float32(scale_x)))] for k in range(d)] for b in range(B)]
     posset = {(int(r), int(c)) for r, c in labels}
     g = [[0.0] * B for _ in range(L)]
     zs = np.float32(scale_w) * np.float32(scale_x)
@@ -295,5 +301,5 @@ def scalar_fp8_step_tiny(w_codes, x_bf16, labels, lr, scale_w=1.0, scale_x=1.0):
             for b in range(B):
                 acc += g[l][b] * float(x_bf16[b, k])
             t = np.float32(w[l][k] - float(np.float32(np.float32(lr) / np.float32(scale_w))) * float(np.float32(acc)))
-            new[l, k] = C.e4m3_encode(t)
+            new[l, k] = C.e4m3_encode(t, saturate=not simulated)
     return new, gx
