@@ -48,15 +48,12 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-    const int upd_lds = T_HALVES * TUP_XBYTES;   // the two-half variants need more than the default 64 KiB
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_RTN, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_BF16, ROUND_SR_PHILOX, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_RTN, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_PHILOX, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
-    (void)hipFuncSetAttribute((const void*)tiled_update_kernel<W_E4M3, ROUND_SR_FAST, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize, upd_lds);
+    // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
+#define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
+    XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false);
+    XMC_UPD_ATTR(W_E4M3, ROUND_RTN, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, false);
+    XMC_UPD_ATTR(W_E4M3, ROUND_RTN, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, true);
+#undef XMC_UPD_ATTR
   }
   return cached[dev];
 }
@@ -89,11 +86,15 @@ __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4* __restrict
 
 int launch_status() { return hipGetLastError() == hipSuccess ? XMC_OK : XMC_ERR_LAUNCH; }
 
-// xmc_fp8_forward_topk takes the chunks in groups: as many as give at most 2^17 labels (fewer, larger launches), one
-// chunk if it is larger than that by itself
-int topk_group(int rows_per_chunk) { const int g = (1 << 17) / rows_per_chunk; return g < 1 ? 1 : g; }
+// xmc_fp8_forward_topk takes the labels in segments of at most 2^17: as many whole chunks as fit (fewer, larger
+// launches), or, for a chunk that is larger than that by itself, pieces of it of 2^17 rows
+constexpr int TOPK_SEG = 1 << 17;
+int topk_group(int rows_per_chunk) { const int g = TOPK_SEG / rows_per_chunk; return g < 1 ? 1 : g; }
+long long topk_segment_rows(int rows_per_chunk) {
+  return rows_per_chunk > TOPK_SEG ? (long long)TOPK_SEG : (long long)topk_group(rows_per_chunk) * rows_per_chunk;
+}
 size_t topk_zbuf_bytes(int rows_per_chunk) {
-  return ((size_t)BP * topk_group(rows_per_chunk) * rows_per_chunk * 2 + 255) / 256 * 256;
+  return ((size_t)BP * (size_t)topk_segment_rows(rows_per_chunk) * 2 + 255) / 256 * 256;
 }
 
 // The launches of the inference logits, shared by xmc_fp8_forward (operand images in the caller's workspace) and
@@ -209,7 +210,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.nquads = qgrid >> 2;
     p.kmax = (num_tiles + p.nquads - 1) / p.nquads;
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
-        labels_coo, nnz, n_pad, batch, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
+        labels_coo, nnz, n_pad, batch, 0, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
     quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, (size_t)(n_pad + 257) * 4, stream>>>(
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
@@ -278,7 +279,6 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   if (scratch_bytes < xmc_topk_scratch_bytes(rows_per_chunk)) return XMC_ERR_WORKSPACE;
   if (num_labels <= 0 || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
   if (k <= 0 || k > TOPK_MAX || k > num_labels) return XMC_ERR_SHAPE;
-  if (rows_per_chunk > (1 << 18)) return XMC_ERR_RANGE;   // the selection kernel indexes a group of chunks with 18 bits
   if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;
@@ -296,31 +296,28 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
   fp.xq = ws + WS_XQ;
   fp.zscale = scale_w * scale_x;
   const int group = topk_group(rows_per_chunk);
-  const long long group_rows = (long long)group * rows_per_chunk;
+  const long long seg_rows = topk_segment_rows(rows_per_chunk);
   fp.out = zbuf;
-  fp.out_stride = group_rows;
+  fp.out_stride = seg_rows;
   fp.num_labels = num_labels;
   fp.batch = batch;
-  // Every batch row keeps two lists.  Large groups are split between two workgroups per row (one list each), so that
+  // Every batch row keeps two lists.  Large segments are split between two workgroups per row (one list each), so that
   // 128 rows occupy all compute units; small ones go to list 0.  A list without k entries yet is first given a short
   // piece (4,096 logits, which fit the workgroup's candidate store): that leaves k entries whose smallest value bounds
   // the rest.
   int have[2] = {0, 0};
   auto select = [&](const unsigned short* zp, int n, int base, int parts) {
-    topk_chunk_kernel<<<batch * parts, TOPK_NT, 0, stream>>>(zp, group_rows, n, base, k, parts, have[0], have[1], run_val, run_idx);
+    topk_chunk_kernel<<<batch * parts, TOPK_NT, 0, stream>>>(zp, seg_rows, n, base, k, parts, have[0], have[1], run_val, run_idx);
     const int n0 = parts == 2 ? topk_split(n) : n;
     have[0] = have[0] + n0 < k ? have[0] + n0 : k;
     have[1] = have[1] + (n - n0) < k ? have[1] + (n - n0) : k;
   };
-  for (int c = 0; c < num_chunks; c += group) {
-    const long long base = (long long)c * rows_per_chunk;
-    if (base >= num_labels) break;
-    const int n = (int)(num_labels - base < group_rows ? num_labels - base : group_rows);   // padding rows are dropped
-    const int full = n / rows_per_chunk, rest = n - full * rows_per_chunk;                   // whole chunks, rows of the last one
-    fp.tile_begin = c * fp.tiles_per_chunk;
-    fp.tile_end = fp.tile_begin + full * fp.tiles_per_chunk + (rest + FT - 1) / FT;
+  // one segment: the logits of tiles [tile_begin, tile_end) into the scratch buffer, then their n labels from `base` on
+  auto segment = [&](int tile_begin, int tile_end, long long base, int n) {
+    fp.tile_begin = tile_begin;
+    fp.tile_end = tile_end;
     fp.col0 = base;
-    const int tiles = fp.tile_end - fp.tile_begin;
+    const int tiles = tile_end - tile_begin;
     fp8_forward_kernel<<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, FWD_LDS, stream>>>(fp);
     int done = 0;
     if (n > 32768) {          // two workgroups per row
@@ -336,6 +333,24 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
       }
       select(zbuf + done, n - done, (int)base + done, 1);
     }
+  };
+  if (rows_per_chunk <= TOPK_SEG) {
+    for (int c = 0; c < num_chunks; c += group) {
+      const long long base = (long long)c * rows_per_chunk;
+      if (base >= num_labels) break;
+      const int n = (int)(num_labels - base < seg_rows ? num_labels - base : seg_rows);     // padding rows are dropped
+      const int full = n / rows_per_chunk, rest = n - full * rows_per_chunk;                // whole chunks, rows of the last one
+      segment(c * fp.tiles_per_chunk, c * fp.tiles_per_chunk + full * fp.tiles_per_chunk + (rest + FT - 1) / FT, base, n);
+    }
+  } else {
+    for (int c = 0; c < num_chunks; c++)
+      for (int r0 = 0; r0 < rows_per_chunk; r0 += TOPK_SEG) {       // TOPK_SEG is a multiple of the tile height
+        const long long base = (long long)c * rows_per_chunk + r0;
+        if (base >= num_labels) break;
+        long long n = rows_per_chunk - r0 < TOPK_SEG ? rows_per_chunk - r0 : TOPK_SEG;
+        if (n > num_labels - base) n = num_labels - base;
+        segment(c * fp.tiles_per_chunk + r0 / FT, c * fp.tiles_per_chunk + r0 / FT + (int)((n + FT - 1) / FT), base, (int)n);
+      }
   }
   topk_finish_kernel<<<batch, 2 * TOPK_MAX, 0, stream>>>(run_val, run_idx, k, have[0], have[1], (unsigned short*)out_val_bf16, out_idx);
   return launch_status();
@@ -351,9 +366,9 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0 || max_batch <= 0 || max_batch > T_HALVES * BP) return 0;
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
-  const size_t halves = ((size_t)max_batch + BP - 1) / BP;
-  // per batch half G in both orientations; tile_ptr (padded to 64 entries); two loss shares per tile
-  return TW_G + halves * 2 * rows_pad * BP * 2 + (tiles + 1 + 63) / 64 * 64 * 4 + (tiles * 8 + 255) / 256 * 256;
+  const size_t halves = (size_t)tiled_halves(max_batch), pairs = (halves + 1) / 2;
+  // per batch half G in both orientations; tile_ptr per pair of halves (padded to 64 entries); two loss shares per tile
+  return tiled_layout((int)halves).g + halves * 2 * rows_pad * BP * 2 + pairs * ((tiles + 1 + 63) / 64 * 64 * 4) + (tiles * 8 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
@@ -387,23 +402,30 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   const int rows_pad = (rows_per_chunk + TL - 1) / TL * TL;
   const int tiles_per_chunk = rows_pad / TL;
   const int num_tiles = num_chunks * tiles_per_chunk;
-  unsigned short* xb = (unsigned short*)(ws + TW_XB);
-  unsigned short* xT = (unsigned short*)(ws + TW_XT);
-  unsigned* keys = (unsigned*)(ws + TW_KEYS);
-  float* gx_total = (float*)(ws + TW_GX);
-  floatx4* partial = (floatx4*)(ws + TW_PART);
-  const int halves = (batch + BP - 1) / BP;
+  const int halves = tiled_halves(batch), pairs = (halves + 1) / 2;   // halves beyond the batch are zero rows of X
+  const TiledLayout lay = tiled_layout(halves);
+  unsigned short* xb = (unsigned short*)(ws + lay.xb);
+  unsigned short* xT = (unsigned short*)(ws + lay.xt);
+  unsigned* keys = (unsigned*)(ws + lay.keys);
+  float* gx_total = (float*)(ws + lay.gx);
+  floatx4* partial = (floatx4*)(ws + lay.part);
   const size_t g_half = 2 * (size_t)rows_pad * BP;    // elements of one half's G and G^T
-  unsigned short* glb = (unsigned short*)(ws + TW_G);
+  unsigned short* glb = (unsigned short*)(ws + lay.g);
   unsigned short* gbl = glb + (size_t)rows_pad * BP;
   int* tile_ptr = (int*)(glb + halves * g_half);
-  float* loss_part = (float*)(tile_ptr + (num_tiles + 1 + 63) / 64 * 64);   // one share per sub-tile of 32 rows
+  const size_t tp_stride = (size_t)(num_tiles + 1 + 63) / 64 * 64;   // entries of one pair's tile_ptr
+  float* loss_part = (float*)(tile_ptr + pairs * tp_stride);         // one share per sub-tile of 32 rows
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
-  if (n_pad > 0)
-    quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, keys, nullptr);
-  tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys, n_pad, rows_per_chunk, tiles_per_chunk, num_tiles, tile_ptr);
+  // the positives of every 256 batch rows as their own sorted list (the key keeps eight bits for the row)
+  for (int pr = 0; pr < pairs; pr++) {
+    if (n_pad > 0)
+      quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, 256 * pr,
+                                                                            keys + (size_t)pr * MAX_POS, nullptr);
+    tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys + (size_t)pr * MAX_POS, n_pad, rows_per_chunk, tiles_per_chunk,
+                                                                  num_tiles, tile_ptr + pr * tp_stride);
+  }
   tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT,
                                                                         gx_total, loss_part, loss_out ? 2 * num_tiles : 0);
   for (int c = 0; c < num_chunks; c++) {
@@ -417,61 +439,66 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     int range = (rp + T_SPLITS - 1) / T_SPLITS;
     range = (range + TL - 1) / TL * TL;
     const int splits = (rp + range - 1) / range;
-    const int* tp = tile_ptr + c * tiles_per_chunk;
     float* lp = loss_part + 2 * c * tiles_per_chunk;
     for (int hh = 0; hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
       unsigned short* gb = gbl + hh * g_half;
       const unsigned short* xh = xb + (size_t)hh * BP * D;
-      const unsigned brow0 = (unsigned)(hh * BP);
+      const unsigned* kh = keys + (size_t)(hh >> 1) * MAX_POS;                       // this half's pair: its keys,
+      const int* tp = tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk;       // its tile_ptr,
+      const unsigned brow0 = (unsigned)((hh & 1) * BP);                             // the half's first row within the pair
+      const int pbatch = batch - 256 * (hh >> 1);                                   // and the batch rows the pair has
       const int nsub = 2 * tiles;                                   // sub-tiles of 32 label rows
       const int lgrid = nsub < di.cus ? nsub : di.cus;              // persistent: one workgroup per compute unit
       if (weight_type == W_BF16) {
-        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
       } else {
-        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
-        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, keys, tp, label0, gl, gb, batch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
       }
     }
-    // grad_X of the chunk: one pass over W for both batch halves, then the fixed-order sums per half
+    // grad_X of the chunk: one pass over W per pair of batch halves, then the fixed-order sums per half
     const size_t part_half = (size_t)T_SPLITS * 4 * 24 * 256;   // floatx4 elements of one half's partials
-    if (weight_type == W_BF16) {
-      if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * splits, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
-      else tiled_gradx_kernel<W_BF16, 2><<<4 * splits, 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
-    } else {
-      if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * splits, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
-      else tiled_gradx_kernel<W_E4M3, 2><<<4 * splits, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gbl, g_half, partial, part_half);
+    for (int h0 = 0; h0 < halves; h0 += 2) {
+      const unsigned short* gsrc = gbl + h0 * g_half;
+      floatx4* pdst = partial + h0 * part_half;
+      if (weight_type == W_BF16) {
+        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * splits, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_BF16, 2><<<4 * splits, 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+      } else {
+        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * splits, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_E4M3, 2><<<4 * splits, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+      }
     }
-    const int ugrid = TRED_WAVES / 4 + 4 * ((tiles + TUP_TILES * halves - 1) / (TUP_TILES * halves));
+    const int nsub_u = tup_threads(halves) / 256;    // tiles a workgroup of the update kernel works on at a time
+    const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) +
+                      (12 / tup_csteps(halves)) * ((tiles + TUP_TILES * nsub_u - 1) / (TUP_TILES * nsub_u));
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
-  tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, 256 * HV, (size_t)TUP_XBYTES * HV, stream>>>(                             \
+  tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV), stream>>>(                           \
       w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0, partial, part_half, splits,           \
       weight_type == W_BF16 ? 1 : 0, gx_total)
-#define XMC_LAUNCH_UPDATE(WTYPE, RMODE)                                                                                        \
+#define XMC_LAUNCH_UPDATE_H(WTYPE, RMODE, KH)                                                                                  \
   do {                                                                                                                         \
-    if (halves == 1) XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 1, false); else XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 2, false);            \
-  } while (0)
-#define XMC_LAUNCH_UPDATE_HEAD(RMODE)                                                                                          \
-  do {                                                                                                                         \
-    if (halves == 1) XMC_LAUNCH_UPDATE_K(W_E4M3, RMODE, 1, true); else XMC_LAUNCH_UPDATE_K(W_E4M3, RMODE, 2, true);            \
+    if (halves == 1) XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 1, KH);                                                                 \
+    else if (halves == 2) XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 2, KH);                                                            \
+    else XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 4, KH);                                                                             \
   } while (0)
     const bool with_head = kahan_type != 0 && nh > 0;   // only chunk 0 of the head-Kahan layer
     if (weight_type == W_BF16) {
-      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_BF16, ROUND_RTN);
-      else XMC_LAUNCH_UPDATE(W_BF16, ROUND_SR_PHILOX);
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_RTN, false);
+      else XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_SR_PHILOX, false);
     } else if (with_head) {
-      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_HEAD(ROUND_RTN);
-      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE_HEAD(ROUND_SR_FAST);
-      else XMC_LAUNCH_UPDATE_HEAD(ROUND_SR_PHILOX);
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_RTN, true);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_SR_FAST, true);
+      else XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_SR_PHILOX, true);
     } else {
-      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_RTN);
-      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_FAST);
-      else XMC_LAUNCH_UPDATE(W_E4M3, ROUND_SR_PHILOX);
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_RTN, false);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_SR_FAST, false);
+      else XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_SR_PHILOX, false);
     }
-#undef XMC_LAUNCH_UPDATE_HEAD
+#undef XMC_LAUNCH_UPDATE_H
 #undef XMC_LAUNCH_UPDATE_K
-#undef XMC_LAUNCH_UPDATE
   }
   tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
   if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, 2 * num_tiles, loss_out);

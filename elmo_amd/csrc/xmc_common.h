@@ -21,7 +21,7 @@ constexpr int TL = 64;            // labels per tile of the training kernels
 constexpr int NT = 256;           // threads per workgroup of the inference kernel (4 wavefronts of 64)
 constexpr int WS = D + 16;        // LDS row stride of a W tile in the inference kernel, bytes (49 x 16)
 constexpr int MAX_CHUNKS = 64;
-constexpr int MAX_POS = 16384;    // positives per step the single-workgroup sort handles
+constexpr int MAX_POS = 32768;    // positives per step (per 256 batch rows on the tiled path): the rank sort keeps them all in LDS
 
 // workspace of the fused step (byte offsets), all 256-byte aligned
 constexpr int MAX_WG = 256;                                   // workgroups of the persistent step kernel

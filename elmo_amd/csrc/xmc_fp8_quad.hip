@@ -153,12 +153,13 @@ __device__ __forceinline__ QTile q_desc_full(q_cdesc* desc, int t) {
 }
 
 // First of the two launches in front of the step kernel: clear the counters (flags, may be null) and sort the positives
-// (key = label*256 + batch row, invalid entries -> 0xFFFFFFFF) by rank.  Workgroup b ranks keys 64b..64b+63 of the n_pad
+// (key = label*256 + (batch row - row0) for the batch rows row0..row0+255 that lie below `batch`; every other entry, and
+// labels outside the label space, -> 0xFFFFFFFF) by rank.  Workgroup b ranks keys 64b..64b+63 of the n_pad
 // (a power of two, at least 64, or 0): every workgroup builds all keys in LDS, its four wavefronts each count the keys
 // that precede the workgroup's own over a quarter of the set (equal keys: the one that comes first in the input
 // precedes), and the sum of the four counts is the key's position in the output.  Grid: max(1, n_pad / 64) x 256
 // threads, (n_pad + 256) * 4 bytes of LDS.
-__global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, unsigned* keys, int* flags) {
+__global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, int row0, unsigned* keys, int* flags) {
   extern __shared__ unsigned sk[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   if (blockIdx.x == 0 && flags)
@@ -176,8 +177,8 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
 #pragma unroll
     for (int u = 0; u < 8; u++) {
       const int i = i0 + u * 256;
-      const int r = e[u].x, lab = e[u].y;
-      if (i < n_pad) sk[i] = (r >= 0 && r < batch && lab >= 0 && lab < (1 << 24) - 1) ? (((unsigned)lab << 8) | (unsigned)r) : 0xFFFFFFFFu;
+      const int r = e[u].x - row0, lab = e[u].y;
+      if (i < n_pad) sk[i] = (r >= 0 && r < 256 && r + row0 < batch && lab >= 0 && lab < (1 << 24) - 1) ? (((unsigned)lab << 8) | (unsigned)r) : 0xFFFFFFFFu;
     }
   }
   __syncthreads();

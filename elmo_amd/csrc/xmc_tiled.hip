@@ -19,16 +19,30 @@ constexpr int T_WS2 = 48 * 2 + 16;                 // LDS row stride of a wavefr
 typedef short tshortx4 __attribute__((ext_vector_type(4)));
 typedef short tshortx8 __attribute__((ext_vector_type(8)));
 
-// The batch is processed in halves of up to 128 rows (T_HALVES of them at most): logits and grad_X per half, grad_W summed
-// over the halves.
-constexpr int T_HALVES = 2;
-// workspace of the tiled path (byte offsets, 256-byte aligned)
-constexpr size_t TW_XB = 0;                                        // X   [halves][128][768] bf16, rows beyond the batch zero
-constexpr size_t TW_XT = TW_XB + (size_t)T_HALVES * BP * D * 2;    // X^T [halves][768][128] bf16
-constexpr size_t TW_KEYS = TW_XT + (size_t)T_HALVES * BP * D * 2;  // sorted positive keys
-constexpr size_t TW_GX = TW_KEYS + (size_t)MAX_POS * 4;            // grad_X total, fp32 [halves*128][768]
-constexpr size_t TW_PART = TW_GX + (size_t)T_HALVES * BP * D * 4;  // grad_X partials [halves][T_SPLITS][128*768] fp32
-constexpr size_t TW_G = TW_PART + (size_t)T_HALVES * T_SPLITS * BP * D * 4;   // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr
+// The batch is processed in halves of up to 128 rows (1, 2 or 4 of them: up to 512 rows): logits per half, grad_X per
+// pair of halves, grad_W summed over all halves in the update kernel.
+constexpr int T_HALVES = 4;
+__host__ __device__ inline int tiled_halves(int batch) { return batch <= BP ? 1 : batch <= 2 * BP ? 2 : 4; }
+// workspace of the tiled path for `halves` batch halves (byte offsets, 256-byte aligned)
+struct TiledLayout {
+  size_t xb;     // X   [halves][128][768] bf16 in operand order, rows beyond the batch zero
+  size_t xt;     // X^T [halves][768][128] bf16 in operand order
+  size_t keys;   // sorted positive keys, one list of MAX_POS entries per pair of halves (key = label*256 + row in the pair)
+  size_t gx;     // grad_X total, fp32 [halves*128][768]
+  size_t part;   // grad_X partials [halves][T_SPLITS][128*768] fp32
+  size_t g;      // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr per pair, loss shares
+};
+inline TiledLayout tiled_layout(int halves) {
+  TiledLayout l;
+  const size_t pairs = (size_t)(halves + 1) / 2;
+  l.xb = 0;
+  l.xt = l.xb + (size_t)halves * BP * D * 2;
+  l.keys = l.xt + (size_t)halves * BP * D * 2;
+  l.gx = l.keys + pairs * MAX_POS * 4 + 256;      // the kernels read up to seven keys past the end of a list
+  l.part = l.gx + (size_t)halves * BP * D * 4;
+  l.g = l.part + (size_t)halves * T_SPLITS * BP * D * 4;
+  return l;
+}
 
 __device__ __forceinline__ bf16x8 t_fp8x8_to_bf16x8(intx2 raw) {
   bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, false), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw.x, 1.0f, true);
@@ -529,22 +543,29 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
 }
 
 constexpr int TUP_TILES = 4;                       // tiles of 64 label rows that each group of four wavefronts processes
-constexpr int TUP_XBYTES = 12 * (BP / 32) * 1024;  // the X^T operand blocks of one feature quarter and batch half: 48 KiB
+// A workgroup owns CS steps of 64 features (CS = 3: a feature quarter, with one or two batch halves; CS = 1: 64 features,
+// with four halves) and keeps their X^T operand blocks of every batch half in LDS: 16 KiB per step and half.
+constexpr int tup_csteps(int halves) { return halves <= 2 ? 3 : 1; }
+constexpr int tup_xbytes(int halves) { return tup_csteps(halves) * 4 * (BP / 32) * 1024; }
+constexpr int tup_threads(int halves) { return halves == 1 ? 256 : 512; }
+constexpr int tup_lds_bytes(int halves) { return halves * tup_xbytes(halves); }
 
-// Launched with 256 threads per batch half and TUP_XBYTES of LDS per batch half: four wavefronts per tile, so that a
-// compute unit runs at least eight wavefronts with one batch half as with two (one workgroup, two tiles at a time).
-// HALVES (batch halves, 1 or 2) and KAHAN (a compensated head may be present) are template parameters: with run-time
+// Launched with tup_threads(HALVES) threads and tup_lds(HALVES) bytes of LDS: four wavefronts per tile, so that a
+// compute unit runs at least eight wavefronts with one batch half (three workgroups) as with more (one workgroup of
+// eight wavefronts, two tiles at a time).
+// HALVES (batch halves: 1, 2 or 4) and KAHAN (a compensated head may be present) are template parameters: with run-time
 // branches around the products the compiler issued every LDS operand read right in front of its matrix instruction.
 template <int WT, int MODE, int HALVES, bool KAHAN>
-__global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_update_kernel(
+__global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES == 2 ? 2 : 1) void tiled_update_kernel(
     void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, unsigned seed,
     int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
     int red_splits, int red_round_bf16, float* red_total) {
   static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
   // the first workgroups sum the chunk's grad_X partials (384 wavefronts per batch half), the others update the weights
-  constexpr int RED_BLOCKS = TRED_WAVES * HALVES / (4 * HALVES);
+  constexpr int CS = tup_csteps(HALVES), XB = tup_xbytes(HALVES), NFB = 12 / CS, WAVES = tup_threads(HALVES) / 64;
+  constexpr int RED_BLOCKS = TRED_WAVES * HALVES / WAVES;
   if ((int)blockIdx.x < RED_BLOCKS) {
-    const int widx = (int)blockIdx.x * (4 * HALVES) + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
+    const int widx = (int)blockIdx.x * WAVES + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
     tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_splits, red_round_bf16,
                       red_total + (size_t)hh * BP * D);
     return;
@@ -553,21 +574,21 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = (tid >> 6) & 3, sub = tid >> 8, nsub = (int)blockDim.x >> 8;
   const int lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fb = ((int)blockIdx.x - RED_BLOCKS) & 3, group = ((int)blockIdx.x - RED_BLOCKS) >> 2;
-  // The X^T operand of this feature quarter goes to LDS once (it is contiguous in the image) and serves all tiles and
+  const int fb = ((int)blockIdx.x - RED_BLOCKS) % NFB, group = ((int)blockIdx.x - RED_BLOCKS) / NFB;   // fb: CS steps of 64 features
+  // The X^T operand of these features goes to LDS once (it is contiguous in the image) and serves all tiles and
   // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
 #pragma unroll
   for (int hh = 0; hh < HALVES; hh++) {
-    const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (TUP_XBYTES / 2));
-    for (int s = tid; s < TUP_XBYTES / 16; s += (int)blockDim.x)
-      *(__attribute__((address_space(3))) intx4*)(lds + hh * TUP_XBYTES + s * 16) = src[s];
+    const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (XB / 2));
+    for (int s = tid; s < XB / 16; s += (int)blockDim.x)
+      *(__attribute__((address_space(3))) intx4*)(lds + hh * XB + s * 16) = src[s];
   }
   __syncthreads();
   // The G rows and the weights of the next tile are loaded before the products of the current one: a wavefront waits
   // for memory once per launch, not four times per tile.
   constexpr int WDW = WT == W_BF16 ? 8 : 4;   // dwords of 16 weights
   bf16x8 gf_n[HALVES][4];
-  intx4 wr_n[3][WDW / 4];
+  intx4 wr_n[CS][WDW / 4];
   auto load_tile = [&](int tile) {
     const int row = tile * TL + 16 * wv + l16;
     const bool live = tile < ntiles && row < rows;
@@ -577,8 +598,8 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
       for (int ks = 0; ks < 4; ks++)
         gf_n[hh][ks] = tile < ntiles ? *(const bf16x8*)(glb + hh * g_half_stride + ((size_t)((tile * 4 + wv) * 4 + ks) * 64 + lane) * 8) : bf16x8{};
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
-      const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 192 * fb + 64 * c + 16 * kg) * (WT == W_BF16 ? 2 : 1));
+    for (int c = 0; c < CS; c++) {
+      const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 64 * (CS * fb + c) + 16 * kg) * (WT == W_BF16 ? 2 : 1));
 #pragma unroll
       for (int q = 0; q < WDW / 4; q++) wr_n[c][q] = live ? src[q] : intx4{0, 0, 0, 0};
     }
@@ -593,19 +614,19 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
   const bool head = KAHAN && kahan_type != 0 && row < num_head;
   const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
   bf16x8 gf[HALVES][4];
-  intx4 wr_t[3][WDW / 4];
+  intx4 wr_t[CS][WDW / 4];
 #pragma unroll
   for (int hh = 0; hh < HALVES; hh++)
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) gf[hh][ks] = gf_n[hh][ks];
 #pragma unroll
-  for (int c = 0; c < 3; c++)
+  for (int c = 0; c < CS; c++)
 #pragma unroll
     for (int q = 0; q < WDW / 4; q++) wr_t[c][q] = wr_n[c][q];
   if (tt + 1 < TUP_TILES) load_tile(tile + nsub);
 #pragma unroll
-  for (int c = 0; c < 3; c++) {               // 16 consecutive features of this lane's row at a time
-    const int col0 = 192 * fb + 64 * c + 16 * kg;
+  for (int c = 0; c < CS; c++) {              // 16 consecutive features of this lane's row at a time
+    const int col0 = 64 * (CS * fb + c) + 16 * kg;
     const size_t idx = (size_t)row * D + col0;
     unsigned wr[WDW], wo[WDW], kr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, ko[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -628,7 +649,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
     // the four 16-feature products of this step: sixteen operand reads in flight (a batch of four or two products),
     // then their matrix instructions
     floatx4 acc[4];
-    constexpr int QB = HALVES == 1 ? 4 : 2;
+    constexpr int QB = HALVES == 1 ? 4 : HALVES == 2 ? 2 : 1;
 #pragma unroll
     for (int q0 = 0; q0 < 4; q0 += QB) {
       bf16x8 xa[QB][HALVES][4];
@@ -638,7 +659,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 3 : 2) void tiled_updat
         for (int hh = 0; hh < HALVES; hh++)
 #pragma unroll
           for (int ks = 0; ks < 4; ks++)
-            xa[qq][hh][ks] = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * TUP_XBYTES +
+            xa[qq][hh][ks] = *(const __attribute__((address_space(3))) bf16x8*)(lds + hh * XB +
                                                                                 (((4 * c + q0 + qq) * (BP / 32) + ks) * 64 + lane) * 16);
 #pragma unroll
       for (int qq = 0; qq < QB; qq++) {

@@ -33,7 +33,7 @@ __device__ __forceinline__ unsigned short topk_bits(unsigned key) {
   return (key & 0x8000u) ? (unsigned short)(key & 0x7FFFu) : (unsigned short)(~key & 0xFFFFu);
 }
 
-// z: a row's logits of the chunk at z + row*stride, n_all of them valid (n_all < 2^18; stride % 4 == 0; z 8-byte aligned)
+// z: a row's logits of the chunk at z + row*stride, n_all of them valid (n_all <= 2^17; stride % 4 == 0; z 8-byte aligned)
 // run_val/run_idx: [batch][2][TOPK_MAX] entries kept so far: every batch row has two lists, which topk_finish_kernel
 // merges.  parts = 1: one workgroup per row adds all n_all logits to list 0 (have0 entries valid).  parts = 2: two
 // workgroups per row, so that 128 rows fill 256 compute units; workgroup 2 row + p takes the first topk_split(n_all)

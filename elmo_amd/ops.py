@@ -7,7 +7,7 @@ from . import _lib
 
 FEATURES = 768
 MAX_BATCH = 128          # fused step
-MAX_BATCH_TILED = 256    # three-kernel step
+MAX_BATCH_TILED = 512    # three-kernel step: up to four halves of 128 rows
 
 
 def _stream_ptr():
@@ -187,7 +187,7 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
         assert c.shape[0] == rows_per_chunk or (i == nc - 1 and 0 < c.shape[0] <= rows_per_chunk)
         arr[i] = c.data_ptr()
     batch = x.shape[0]
-    assert 0 < batch <= MAX_BATCH_TILED, "batch must be at most 256"
+    assert 0 < batch <= MAX_BATCH_TILED, "batch must be at most 512"
     if workspace is None or workspace.numel() < tiled_workspace_bytes(nc, rows_per_chunk, batch):
         workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device, batch)
     if grad_out is None:

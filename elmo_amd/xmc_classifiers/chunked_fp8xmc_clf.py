@@ -87,7 +87,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self._err_dev = self._workspace[off:off + 4].view(torch.int32)
         self._err_host = torch.zeros(1, dtype=torch.int32).pin_memory()
         self._err_event = None
-        # batches of more than 128 rows (up to 256) also run on the three-kernel path, with the true-FP8 arithmetic
+        # batches of more than 128 rows (up to 512) also run on the three-kernel path, with the true-FP8 arithmetic
         self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "simulated FP8 has no per-tensor scales"
@@ -146,7 +146,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         '''
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args:
-            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 256 (the fused
+            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 512 (the fused
                    kernel takes up to 128 rows, larger batches run on the three-kernel path).
             labels: Positive labels in sparse format, int32 [Nb, 2] = (row in batch, label id).
             xmc_lr: list of learning rates, only [0] is used.
@@ -154,7 +154,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         '''
         assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
         assert embed.shape[0] <= ops.MAX_BATCH_TILED and (self.fake_fp8_matmul or embed.shape[0] % 16 == 0), \
-            "batch must be a multiple of 16 and at most 256 (the reference data loader uses drop_last)"
+            "batch must be a multiple of 16 and at most 512 (the reference data loader uses drop_last)"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
         x = embed.detach()
         if x.dtype != torch.bfloat16:

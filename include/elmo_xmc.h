@@ -97,8 +97,9 @@ int xmc_fp8_forward_static(void* const* chunk_ptrs, int num_chunks, int rows_per
                            int features, float scale_w, float scale_x, void* out_bf16, long long out_stride,
                            long long num_labels, void* stream);
 
-/* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one group of chunks (up to 2^17 labels, or one
- * chunk of up to 2^18 rows) and the running lists (two of 128 entries per batch row). */
+/* Bytes of the scratch buffer of xmc_fp8_forward_topk: the logits of one segment of labels (as many whole chunks as
+ * give at most 2^17 labels, or a 2^17-row piece of a larger chunk) and the running lists (two of 128 entries per batch
+ * row).  Any rows_per_chunk that is a multiple of 16. */
 size_t xmc_topk_scratch_bytes(int rows_per_chunk);
 
 /* Inference with the top-k taken chunk by chunk: what the evaluation loop computes as
@@ -124,7 +125,7 @@ enum {
   XMC_WEIGHT_BF16 = 1       /* bf16 layer (chunked.py:85-131) */
 };
 
-/* Bytes of workspace xmc_tiled_step needs for batches of up to max_batch rows (1..256). */
+/* Bytes of workspace xmc_tiled_step needs for batches of up to max_batch rows (1..512). */
 size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_batch);
 
 /* One training step of the modes in which the reference keeps bf16 temporaries, three kernels per chunk as there:
@@ -138,7 +139,7 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
  *   round_mode       XMC_ROUND_RTN, XMC_ROUND_SR_PHILOX, or (e4m3 weights only) XMC_ROUND_SR_FAST with the random words of
- *                    xmc_fp8_step's mode of that name; batch: 1..256, any value (processed in halves of 128 rows)
+ *                    xmc_fp8_step's mode of that name; batch: 1..512, any value (processed in one, two or four halves of 128 rows)
  *   quantize_x       e4m3 weights: 0 = logits from the un-quantised X (simulated FP8), 1 = from e4m3(X) (true FP8, :101)
  *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
  *   kahan, kahan_type, num_head

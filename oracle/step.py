@@ -247,6 +247,44 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
     return out + (parts,) if return_parts else out
 
 
+def dense_step(w, x, labels, lr, wd, num_chunks, dtype="float32"):
+    """One step of the fp32 / fp16 branch of the `chunked` layer (chunked.py:85-124): everything in the weight's type,
+    weight decay folded into the gradient, plain SGD.
+        Z = cast(X W_c^T); S = cast(sigmoid(Z)); G = S, cast(S - 1) at positives (set semantics)        :101-113
+        gX += f32(cast(G W_c))                                                                         :116
+        A = cast(G^T X); A = cast(A + wd*W_c); W_c = cast(W_c - lr*A)                                  :119-124
+    cast = round to the weight's type (float32: the float64 sums rounded once; float16: rounded to half).  wd and lr
+    enter as Python floats (torch's alpha): the elementwise results are computed in fp32 and rounded once.
+    Returns (new_w, gx_fp32, grad_input in the weight's type, held in fp32)."""
+    assert dtype in ("float32", "float16")
+    cast = (lambda a: np.asarray(a, dtype=np.float64).astype(np.float32)) if dtype == "float32" else \
+           (lambda a: np.asarray(a, dtype=np.float64).astype(np.float16).astype(np.float32))
+    w_all = cast(w)
+    xc = cast(x)
+    B, d = xc.shape
+    L = w_all.shape[0]
+    cs = (L + num_chunks - 1) // num_chunks
+    x64 = xc.astype(np.float64)
+    gx = np.zeros((B, d), dtype=np.float32)
+    new_w = w_all.copy()
+    for c in range(num_chunks):
+        lo, hi = c * cs, min((c + 1) * cs, L)
+        if lo >= hi:
+            continue
+        w64 = w_all[lo:hi].astype(np.float64)
+        z = cast(x64 @ w64.T)
+        pos = _positives_mask(labels, B, lo, hi).T
+        s = cast(1.0 / (1.0 + np.exp(-z.astype(np.float64))))
+        g = np.where(pos, cast(s.astype(np.float64) - 1.0), s).astype(np.float32)
+        g64 = g.astype(np.float64)
+        gx = (gx + cast(g64 @ w64)).astype(np.float32)
+        a = cast(g64.T @ x64)
+        # torch's add_(other, alpha): self + alpha*other evaluated in fp32 and rounded to the tensor's type
+        a = cast((a.astype(np.float32) + np.float32(wd) * w_all[lo:hi]).astype(np.float32))
+        new_w[lo:hi] = cast((w_all[lo:hi] + np.float32(-lr) * a).astype(np.float32))
+    return new_w, gx, cast(gx)
+
+
 def bce_loss_sum(z_bf16, posmask):
     """Summed binary cross entropy with logits, the quantity chunked.py:57-72 is written to return when it is handed
     the logits: sum(max(z,0)) - sum(z at positives) + sum(log(1 + exp(-|z|))).  float64; z are the bf16 logits."""

@@ -108,3 +108,30 @@ def test_topk_when_most_logits_tie(gpu, k, nc):
     vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k)
     want_v, want_i = O.topk_of_logits(dense, k)
     assert np.array_equal(vals.float().cpu().numpy(), want_v) and np.array_equal(idx.cpu().numpy(), want_i)
+
+
+def test_topk_at_the_shipped_670k_geometry(gpu):
+    """amazontitles670k.yaml ships num_chunks: 2, i.e. chunks of 335,056 rows: larger than one selection segment, so each
+    chunk is taken in three pieces.  Against torch.topk of the library's own dense logits (values bit-equal; ids point at
+    those values and agree wherever the value is unique in its row)."""
+    import torch
+    from elmo_amd import ops
+    L, nc, k, batch = 670091, 2, 100, 16
+    rows = (L + 16 * nc - L % (16 * nc)) // nc
+    assert rows == 335056 and rows > (1 << 18)
+    gen = torch.Generator(device=gpu).manual_seed(12)
+    chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.3).to(torch.float8_e4m3fn) for _ in range(nc)]
+    x = torch.from_numpy(synth.make_x(batch, 768, 13)).to(gpu).to(torch.bfloat16)
+    dense = ops.fp8_forward(chunks, x, L)
+    vals, idx = ops.fp8_forward_topk(chunks, x, L, k)
+    tv, ti = torch.topk(dense.float(), k, dim=1)
+    assert torch.equal(vals.float(), tv)
+    assert torch.equal(dense.float().gather(1, idx), tv) and int(idx.max()) < L and int(idx.min()) >= 0
+    # the documented order among equal values: ascending label id
+    v, i = vals.float().cpu().numpy(), idx.cpu().numpy()
+    tie = v[:, 1:] == v[:, :-1]
+    assert np.all(i[:, 1:][tie] > i[:, :-1][tie])
+    uniq = np.ones_like(v, dtype=bool); uniq[:, 1:] &= ~tie; uniq[:, :-1] &= ~tie
+    assert np.array_equal(i[uniq], ti.cpu().numpy()[uniq])
+    # labels from both chunks and from all three pieces of a chunk appear
+    assert (i >= rows).any() and (i < rows).any()

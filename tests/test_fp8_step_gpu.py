@@ -102,13 +102,13 @@ def test_duplicate_and_dense_positives(gpu):
 
 
 def test_many_positives_boundary_labels_and_ignored_entries(gpu):
-    """Close to the 16,384 pairs a step accepts (the sort and the descriptor search then use their largest LDS
+    """Close to the 32,768 pairs a step accepts (the sort and the descriptor search then use their largest LDS
     footprint), with positives on the first and last label, on both sides of the chunk boundary and in every batch
     row; pairs whose row or label lies outside the batch or the label space are ignored."""
     nc, rows, batch = 2, 4096, 128
     L = nc * rows
     rng = np.random.default_rng(77)
-    flat = rng.choice(batch * L, size=16000, replace=False)
+    flat = rng.choice(batch * L, size=32000, replace=False)
     valid = np.stack([flat // L, flat % L], axis=1).astype(np.int32)
     edge = np.array([[0, 0], [127, L - 1], [5, rows - 1], [5, rows], [64, rows - 1], [0, L - 1]], dtype=np.int32)
     valid = np.concatenate([valid, edge], axis=0)

@@ -303,3 +303,43 @@ def test_topk_matches_the_library_routine():
     tiny = np.array([[1.0, 3.0, 3.0, 2.0]], dtype=np.float32)
     v, i = O.topk_of_logits(tiny, 3)
     assert v.tolist() == [[3.0, 3.0, 2.0]] and i.tolist() == [[1, 2, 3]]
+
+
+@pytest.mark.parametrize("dtype,tdt", [("float32", torch.float32), ("float16", torch.float16)])
+def test_dense_step_matches_torch_cpu(dtype, tdt):
+    """The fp32 / fp16 branch of the `chunked` layer is plain torch in the reference (chunked.py:97-124), so the oracle's
+    restatement is held to those very operations on the CPU: weights within one unit of the type's last place where the
+    GEMM sums differ in their last bits, mostly identical; weight decay visibly applied."""
+    rng = np.random.default_rng(9)
+    L, d, B, nc, lr, wd = 150, 48, 12, 4, 0.05, 0.5
+    w = (rng.standard_normal((L, d)) * 0.05).astype(np.float32)
+    x = synth.make_x(B, d, 9)
+    labels = synth.make_labels(B, L, 3.0, 1.0, 9)
+    labels = np.concatenate([labels, labels[:2]])                     # duplicates count once
+    new, gx, gi = O.dense_step(w, x, labels, lr, wd, nc, dtype)
+    wt = torch.from_numpy(w).to(tdt).clone()
+    xt = torch.from_numpy(x).to(tdt)
+    rows, cols = torch.from_numpy(labels[:, 0].astype(np.int64)), torch.from_numpy(labels[:, 1].astype(np.int64))
+    gt = torch.zeros(B, d)
+    cs = (L + nc - 1) // nc
+    for c in range(nc):
+        lo, hi = c * cs, min((c + 1) * cs, L)
+        wc = wt[lo:hi]
+        out = torch.matmul(xt, wc.t())
+        m = (cols >= lo) & (cols < hi)
+        torch.sigmoid(out, out=out)
+        out[rows[m], cols[m] - lo] -= 1.0
+        gt += torch.matmul(out, wc)
+        grad = out.t().mm(xt)
+        grad.add_(wc, alpha=wd)
+        wc.add_(grad, alpha=-lr)
+    got_w = wt.float().numpy()
+    ulp = 2.0 ** -23 if dtype == "float32" else 2.0 ** -10
+    assert np.all(np.abs(new - got_w) <= 4 * ulp * np.maximum(np.abs(new), np.abs(w).max()))
+    # (a last-place difference in one logit moves a whole row of grad_W by less than its rounding step, which still flips
+    # some of the row's roundings: identical entries are the majority, not all)
+    assert np.mean(new == got_w) > (0.5 if dtype == "float32" else 0.75)
+    assert np.abs(gx - gt.numpy()).max() <= (1e-5 if dtype == "float32" else 2e-3) * np.abs(gx).max()
+    # weight decay is in effect: the same step without it ends elsewhere
+    no_wd, _, _ = O.dense_step(w, x, labels, lr, 0.0, nc, dtype)
+    assert np.abs(no_wd - new).max() > 10 * ulp * np.abs(new).max()

@@ -60,7 +60,9 @@ def check_gx(gf, gb, ref_gx, tol=1e-3):
     (5000, 2, 128, 33),         # full batch
     (20011, 4, 64, 34),         # prime label count
     (3000, 2, 200, 35),         # two batch halves, the second one short
-    (1500, 3, 256, 36),         # the largest batch
+    (1500, 3, 256, 36),         # two full halves
+    (2000, 2, 300, 37),         # three halves (run as four, the last one empty), positives on rows past 256
+    (1300, 3, 512, 38),         # the largest batch: four halves, the batch the reference's chunked configs ship
 ])
 def test_bf16_layer_rtn_parity(gpu, L, nc, batch, seed):
     x, w, labels = bf16_case(L, batch, seed)
@@ -121,6 +123,25 @@ def test_bf16_layer_duplicates_and_no_positives(gpu):
     none = np.zeros((0, 2), dtype=np.int32)
     new, gf, gb = run_bf16(x, w, none, 2, gpu, "rtn", None)
     ref_w, ref_gx, _ = O.bf16_step(w, x, none, 0.05, 2, sr_mode="rtn")
+    check_bf16_weights(new, ref_w, w, x)
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+
+
+def test_bf16_layer_many_positives_over_four_halves(gpu):
+    """30,000 positives (close to the 32,768 a step accepts) spread over 512 batch rows, i.e. over both sorted lists, with
+    pairs on the first and last row of every half; entries outside the batch are ignored."""
+    L, nc, batch = 2048, 2, 512
+    x, w, _ = bf16_case(L, batch, 39)
+    rng = np.random.default_rng(40)
+    flat = rng.choice(batch * L, size=30000, replace=False)
+    labels = np.stack([flat // L, flat % L], axis=1).astype(np.int32)
+    edge = np.array([[r, c] for r in (0, 127, 128, 255, 256, 383, 384, 511) for c in (0, L - 1, 1023, 1024)], dtype=np.int32)
+    labels = np.concatenate([labels, edge])
+    bogus = np.array([[512, 3], [-1, 3], [700, 9], [3, L], [3, -1]], dtype=np.int32)
+    mixed = np.concatenate([labels, bogus])
+    mixed = mixed[rng.permutation(len(mixed))]
+    new, gf, gb = run_bf16(x, w, mixed, nc, gpu, "rtn", None)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.05, nc, sr_mode="rtn")
     check_bf16_weights(new, ref_w, w, x)
     check_gx(gf, gb, ref_gx, tol=4e-3)
 
@@ -210,9 +231,9 @@ def test_chunked_module_contract(gpu):
     _, _, _, ref_loss = O.bf16_step(w1, out2.detach().float().cpu().numpy(), labels.cpu().numpy(), 0.05, 3, sr_mode="rtn",
                                     return_loss=True)
     assert isinstance(loss, float) and abs(loss - ref_loss) <= 1e-4 * abs(ref_loss), (loss, ref_loss)
-    with pytest.raises(AssertionError):
+    with pytest.raises(AssertionError):      # no such weight type in the reference's dtype_map either
         cfg2 = make_cfg("cuda:0", 1000, 3)
-        cfg2.model.xmc.dtype = "float32"
+        cfg2.model.xmc.dtype = "float8"
         XMCBCECHUNKEDLayer(cfg2)
 
 
@@ -433,3 +454,54 @@ def test_tiled_step_replays_in_a_captured_graph(gpu):
         assert torch.equal(gout.view(torch.int16), eager[k][1]), f"grad_input differs after replay {k}"
         scratch = torch.randn(1 << 20, device=gpu).sum().item()      # unrelated eager work between the replays
         assert scratch == scratch
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_chunked_module_fp32_fp16_branch_with_weight_decay(gpu, dtype):
+    """chunked.py:122-124: fp32 / fp16 weights take the plain SGD branch with weight decay, at any batch size (here 300,
+    more than the kernels' 256).  Against the oracle's restatement, which is held to torch CPU operations."""
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked import XMCBCECHUNKEDLayer
+    L, nc, B, lr, wd = 1000, 3, 300, 0.05, 0.5
+    cfg = make_cfg("cuda:0", L, nc)
+    cfg.model.xmc.dtype = dtype
+    cfg.training.xmc.wd = wd
+    cfg.training.precision.mode = "purefp" if dtype == "float32" else "custom"
+    cfg.data.batch_size = B
+    torch.manual_seed(3)
+    xfc = XMCBCECHUNKEDLayer(cfg)
+    tdt = torch.float32 if dtype == "float32" else torch.float16
+    assert xfc._dtype == tdt and xfc.xfc_weight.dtype == tdt and xfc.xfc_weight.shape == (L, 768)
+    w0 = xfc.xfc_weight.float().cpu().numpy().copy()
+    x = synth.make_x(B, 768, 8)
+    labels = synth.make_labels(B, L, 3.0, 1.0, 8)
+    xd = torch.from_numpy(x).to(gpu).to(torch.bfloat16)                  # the encoder hands over bf16; the layer casts (:89-90)
+    ld = torch.from_numpy(labels).to(gpu)
+    loss = xfc.xfc_forward_backward(xd, ld, [lr])
+    assert loss == 0 and xfc.iteration == 1 and xfc.grad_input.dtype == tdt and xfc.grad_input.shape == (B, 768)
+    new, gx, gi = O.dense_step(w0, x, labels, lr, wd, nc, dtype)
+    got = xfc.xfc_weight.float().cpu().numpy()
+    ulp = 2.0 ** -23 if dtype == "float32" else 2.0 ** -10
+    assert np.all(np.abs(new - got) <= 8 * ulp * np.maximum(np.abs(new), np.abs(w0).max()))
+    assert np.abs(xfc.grad_input.float().cpu().numpy() - gi).max() <= (1e-4 if dtype == "float32" else 4e-3) * np.abs(gi).max()
+    # weight decay reached the update
+    nowd, _, _ = O.dense_step(w0, x, labels, lr, 0.0, nc, dtype)
+    assert np.abs(nowd - got).max() > 10 * ulp * np.abs(got).max()
+
+
+@pytest.mark.gpu
+def test_true_fp8_arithmetic_at_batch_512(gpu):
+    """The FP8 layer at the batch its shipped 670K configuration uses twice over (512 rows, four halves on the three-kernel
+    path): logits from e4m3(X), saturating cast, round to nearest - against the true-FP8 oracle."""
+    from elmo_amd import ops
+    case = H.make_case(2, 1024, 512, 64, pos_mean=4.0)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    g, gf = ops.tiled_step(chunks, 1024, "e4m3", x, labels, 0.05, round_mode="rtn", want_f32=True, quantize_x=True, saturate=True)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn")
+    new = H.chunks_to_numpy(chunks)
+    for a, b in zip(new, ref_codes):
+        d = H.e4m3_ulp_distance(a, b)
+        assert d.max() <= 1 and (d != 0).mean() < 5e-3
+    check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx)
