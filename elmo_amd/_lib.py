@@ -64,6 +64,11 @@ def load():
     lib.xmc_fp8_forward_topk.restype = i32
     lib.xmc_fp8_forward_topk.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp, vp,
                                          vp, sz, vp, sz, vp]
+    lib.xmc_topk_fused_scratch_bytes.restype = sz
+    lib.xmc_topk_fused_scratch_bytes.argtypes = []
+    lib.xmc_fp8_forward_topk_fused.restype = i32
+    lib.xmc_fp8_forward_topk_fused.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp,
+                                               vp, vp, sz, vp, sz, vp, vp]
     lib.xmc_step_error_offset.restype = sz
     lib.xmc_step_workgroups.restype = i32
     lib.xmc_step_xcc_ids.restype = i32
@@ -76,6 +81,9 @@ def load():
     lib.xmc_profile_events.argtypes = [vp, vp]
     _lib = lib
     return lib
+
+
+XMC_ERR_RANGE = -4
 
 
 def check(status, what):

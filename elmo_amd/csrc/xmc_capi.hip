@@ -40,6 +40,8 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
+    (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
+    (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
     (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
     (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
     (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2>::LDS);
@@ -353,6 +355,75 @@ int xmc_fp8_forward_topk(void* const* chunk_ptrs, int num_chunks, int rows_per_c
       }
   }
   topk_finish_kernel<<<batch, 2 * TOPK_MAX, 0, stream>>>(run_val, run_idx, k, have[0], have[1], (unsigned short*)out_val_bf16, out_idx);
+  return launch_status();
+}
+
+// scratch of xmc_fp8_forward_topk_fused: group maxima, bounds, counts, candidate labels and keys
+constexpr size_t SELS_GMAX = 0;
+constexpr size_t SELS_BOUND = SELS_GMAX + (size_t)SEL_GROUPS * BP * 2;
+constexpr size_t SELS_COUNT = SELS_BOUND + 256;
+constexpr size_t SELS_LABEL = SELS_COUNT + (size_t)BP * 4;
+constexpr size_t SELS_KEY = SELS_LABEL + (size_t)BP * SEL_CAP * 4;
+constexpr size_t SELS_BYTES = SELS_KEY + (size_t)BP * SEL_CAP * 2;
+static_assert(SEL_CAP == TOPK_LIST && SEL_GROUPS == TOPK_GROUPS, "the two top-k kernels share these sizes");
+
+size_t xmc_topk_fused_scratch_bytes(void) { return SELS_BYTES; }
+
+// tiles pass 1 skips between two it visits: the k-th largest of the group maxima of a 1/step sample leaves about
+// k * step candidates per row, which have to stay well below the list size; at least four groups per wanted entry
+static int topk_fused_step(int tiles, int k) {
+  int step = 16;
+  while (step > 1 && (k * step > SEL_CAP / 2 || tiles / step < 4 * k)) step >>= 1;
+  return tiles / step >= 4 * k ? step : 0;
+}
+
+int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                               int features, float scale_w, float scale_x, long long num_labels, int k, void* out_val_bf16,
+                               int32_t* out_idx, void* workspace, size_t workspace_bytes, void* scratch, size_t scratch_bytes,
+                               int32_t* status, void* stream_) {
+  int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
+  if (st != XMC_OK) return st;
+  if (!out_val_bf16 || !out_idx || !scratch || !status) return XMC_ERR_NULL;
+  if (((uintptr_t)scratch & 255) != 0 || ((uintptr_t)status & 3) != 0) return XMC_ERR_ALIGN;
+  if (scratch_bytes < SELS_BYTES) return XMC_ERR_WORKSPACE;
+  if (num_labels <= 0 || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
+  if (k <= 0 || k > TOPK_MAX || k > num_labels) return XMC_ERR_SHAPE;
+  if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  SelectParams sp;
+  sp.rows_per_chunk = rows_per_chunk;
+  sp.tiles_per_chunk = (rows_per_chunk + FT - 1) / FT;
+  const int last_chunk = (int)((num_labels - 1) / rows_per_chunk);
+  const int tiles = last_chunk * sp.tiles_per_chunk + (int)((num_labels - (long long)last_chunk * rows_per_chunk + FT - 1) / FT);
+  const int step = topk_fused_step(tiles, k);
+  if (step == 0) return XMC_ERR_RANGE;   // too few labels for a useful bound: xmc_fp8_forward_topk takes these
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  unsigned char* ws = (unsigned char*)workspace;
+  unsigned char* sc = (unsigned char*)scratch;
+  prep_x_kernel<<<(BP * (D / 4) + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, 1.0f / scale_x, ws + WS_XQ,
+                                                              (unsigned short*)(ws + WS_XT));
+  for (int c = 0; c < MAX_CHUNKS; c++) sp.chunk[c] = c < num_chunks ? (const unsigned char*)chunk_ptrs[c] : nullptr;
+  sp.xq = ws + WS_XQ;
+  sp.zscale = scale_w * scale_x;
+  sp.num_labels = num_labels;
+  sp.batch = batch;
+  sp.gmax = (unsigned short*)(sc + SELS_GMAX);
+  sp.bound = (const unsigned short*)(sc + SELS_BOUND);
+  sp.count = (unsigned*)(sc + SELS_COUNT);
+  sp.cand_label = (unsigned*)(sc + SELS_LABEL);
+  sp.cand_key = (unsigned short*)(sc + SELS_KEY);
+  // pass 1: the sampled tiles, one group of them per workgroup
+  sp.tile_step = step;
+  sp.n_visit = (tiles + step - 1) / step;
+  const int groups = sp.n_visit < SEL_GROUPS ? sp.n_visit : SEL_GROUPS;
+  fp8_forward_select_kernel<0><<<groups, NT, SEL_LDS, stream>>>(sp);
+  topk_bound_kernel<<<BP, TOPK_GROUPS, 0, stream>>>(sp.gmax, groups, k, batch, (unsigned short*)(sc + SELS_BOUND), sp.count, status);
+  // pass 2: every tile
+  sp.tile_step = 1;
+  sp.n_visit = tiles;
+  fp8_forward_select_kernel<1><<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, SEL_LDS, stream>>>(sp);
+  topk_pick_kernel<<<batch, TOPK_LIST, 0, stream>>>(sp.cand_label, sp.cand_key, sp.count, k, (unsigned short*)out_val_bf16, out_idx, status);
   return launch_status();
 }
 

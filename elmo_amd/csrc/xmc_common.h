@@ -134,4 +134,14 @@ __device__ __forceinline__ unsigned round4(float t0, float t1, float t2, float t
   return (unsigned)packed;
 }
 
+// 16-bit key of a bf16 value for the top-k selection: ascending key order == ascending value order, -0 below +0, and
+// NaN of either sign above everything (torch.topk treats NaN as the largest value), all NaNs alike.
+__device__ __forceinline__ unsigned topk_key(unsigned short bits) {
+  if ((bits & 0x7FFFu) > 0x7F80u) return 0xFFFFu;
+  return (bits & 0x8000u) ? (unsigned)(~bits & 0xFFFFu) : (unsigned)(bits | 0x8000u);
+}
+__device__ __forceinline__ unsigned short topk_bits(unsigned key) {   // key 0xFFFF gives back a NaN (0x7FFF)
+  return (key & 0x8000u) ? (unsigned short)(key & 0x7FFFu) : (unsigned short)(~key & 0xFFFFu);
+}
+
 }  // namespace xmc

@@ -205,4 +205,211 @@ __global__ __launch_bounds__(NT) void fp8_forward_kernel(const ForwardParams p) 
   fp8_forward_body(p, lds_raw, (int)blockIdx.x, (int)gridDim.x);
 }
 
+
+// ---- Top-k of the inference logits without the logits in memory: two passes over the weights.
+// Pass 1 (MODE 0) visits every tile_step-th tile; workgroup g keeps, per batch row, the largest logit of the tiles it
+// visited (its tiles are spread over the whole label range) and writes these maxima as order keys to gmax[g][b].  The
+// k-th largest of a row's maxima is at or below the row's k-th largest logit (k different groups each hold a logit at
+// or above it): topk_bound_kernel stores it as the row's bound.  Pass 2 (MODE 1) visits every tile and appends the
+// logits at or above the bound to the row's candidate list (label and key), in no particular order;
+// topk_pick_kernel ranks the list.  A list holds SEL_CAP entries; the count keeps running past that, and the pick
+// kernel reports a row whose count exceeded it.
+constexpr int SEL_CAP = 1024;
+constexpr int SEL_GROUPS = 512;          // most workgroups of pass 1
+constexpr int SEL_QUEUE = 256;           // candidates a workgroup of pass 2 collects in LDS between two flushes
+constexpr int SEL_FLUSH = 8;             // tiles between two flushes
+constexpr int SEL_LDS = FWD_LDS + 16 + SEL_QUEUE * 8;
+
+struct SelectParams {
+  const unsigned char* chunk[MAX_CHUNKS];
+  int rows_per_chunk, tiles_per_chunk;
+  int n_visit, tile_step;        // the launch visits tiles j * tile_step, j in [0, n_visit)
+  const unsigned char* xq;       // logits operands (prep kernel layout)
+  float zscale;
+  long long num_labels;          // labels at or past this one do not take part
+  int batch;
+  unsigned short* gmax;          // MODE 0: [gridDim.x][BP] keys
+  const unsigned short* bound;   // MODE 1: [BP] keys
+  unsigned* count;               // MODE 1: [BP]
+  unsigned* cand_label;          // MODE 1: [BP][SEL_CAP]
+  unsigned short* cand_key;      // MODE 1: [BP][SEL_CAP]
+};
+
+typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pk_max_u16(unsigned a, unsigned b) {
+  return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(ushortx2, a), __builtin_bit_cast(ushortx2, b)));
+}
+// order keys of two packed bf16 values (topk_key per half, without its NaN rule: a NaN with the sign bit set gets a small key)
+__device__ __forceinline__ unsigned key_pair(unsigned w) {
+  const unsigned s = (w >> 15) & 0x00010001u;
+  return w ^ (((s << 16) - s) | 0x80008000u);   // (s << 16) - s: 0xFFFF in the halves whose sign bit is set
+}
+
+template <int MODE>
+__global__ __launch_bounds__(NT) void fp8_forward_select_kernel(const SelectParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int block = blockIdx.x, nblocks = gridDim.x;
+  const unsigned lds0 = (unsigned)(size_t)(lds_u8*)lds_raw;
+  intx8 xq[2][6];
+#pragma unroll
+  for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++)
+      xq[nb][ks] = *(const intx8*)(p.xq + ((size_t)((w * 2 + nb) * 6 + ks) * 64 + lane) * 32);
+  unsigned bkey[2] = {0xFFFFu, 0xFFFFu}, bm1[2] = {0xFFFEFFFEu, 0xFFFEFFFEu};
+  if (MODE == 1) {
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      const int b = 32 * w + 16 * nb + l16;
+      if (b < p.batch) {
+        unsigned t = p.bound[b];
+        t = t < 1u ? 1u : t;
+        bkey[nb] = t;
+        bm1[nb] = (t - 1u) * 0x00010001u;
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  auto issue = [&](int j, int buf) {
+    const int t = j * p.tile_step;
+    const int c = t / p.tiles_per_chunk, row0 = (t - c * p.tiles_per_chunk) * FT;
+    fwd_issue_tile(p.chunk[c] + (size_t)row0 * D, min(FT, p.rows_per_chunk - row0), lds0 + (unsigned)buf * FB, w, lane);
+  };
+  unsigned mx[2] = {0u, 0u};
+  unsigned* q_cnt = (unsigned*)(lds_raw + FWD_LDS);
+  unsigned long long* q_ent = (unsigned long long*)(lds_raw + FWD_LDS + 16);
+  auto emit = [&](unsigned long long ent) {
+    const unsigned b = (unsigned)(ent >> 48);
+    const unsigned slot = atomicAdd(p.count + b, 1u);
+    if (slot < (unsigned)SEL_CAP) {
+      p.cand_label[(size_t)b * SEL_CAP + slot] = 0xFFFFFFFFu - (unsigned)ent;
+      p.cand_key[(size_t)b * SEL_CAP + slot] = (unsigned short)(ent >> 32);
+    }
+  };
+  int since = 0;
+  if (MODE == 1) {
+    if (tid == 0) *q_cnt = 0u;   // visible to all after the first barrier below
+  }
+  if (block < p.n_visit) {
+    issue(block, 0);
+    if (block + nblocks < p.n_visit) {
+      issue(block + nblocks, 1);
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(FWD_DMA) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int j = block; j < p.n_visit; j += nblocks) {
+      const int t = j * p.tile_step;
+      const int c = t / p.tiles_per_chunk, row0 = (t - c * p.tiles_per_chunk) * FT;
+      const int rows_valid = min(FT, p.rows_per_chunk - row0);
+      const long long label0 = (long long)c * p.rows_per_chunk + row0;
+      const long long left = p.num_labels - label0;
+      const int nvalid = (int)(left < rows_valid ? (left < 0 ? 0 : left) : rows_valid);
+      const unsigned char* wt = lds_raw + buf * FB;
+      const bool more = j + 2 * nblocks < p.n_visit;
+      // the buffer two ahead was read in the iteration before this one, which every wavefront has left (barrier below)
+      if (more) issue(j + 2 * nblocks, buf == 0 ? 2 : buf - 1);
+      floatx4 z[2][2];
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++) { z[rb][0] = floatx4{0.f, 0.f, 0.f, 0.f}; z[rb][1] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+      for (int ks = 0; ks < 6; ks++)
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+          intx8 a = lds_read32(wt + (16 * rb + l16) * WS + ks * 128 + kg * 32);
+          z[rb][0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq[0][ks], z[rb][0], 0, 0, 0, 0, 0, 0);
+          z[rb][1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, xq[1][ks], z[rb][1], 0, 0, 0, 0, 0, 0);
+        }
+      // a lane holds, for batch rows 32w + 16nb + l16, the logits of tile rows 16rb + 4kg + e (e = 0..3): the bf16
+      // values the dense kernel would store, two to a word
+      unsigned wp[2][2][2];
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+          wp[rb][nb][0] = bf16_pack2(z[rb][nb][0] * p.zscale, z[rb][nb][1] * p.zscale);
+          wp[rb][nb][1] = bf16_pack2(z[rb][nb][2] * p.zscale, z[rb][nb][3] * p.zscale);
+        }
+      if (MODE == 0) {
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int hw = 0; hw < 2; hw++) {
+              unsigned kw = key_pair(wp[rb][nb][hw]);
+              if (nvalid < FT) {   // rows past the end of the chunk or of the labels do not count
+                const int r = 16 * rb + 4 * kg + 2 * hw;
+                kw &= (r < nvalid ? 0x0000FFFFu : 0u) | (r + 1 < nvalid ? 0xFFFF0000u : 0u);
+              }
+              mx[nb] = pk_max_u16(mx[nb], kw);
+            }
+      } else {
+        unsigned any = 0u, mag = 0u;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+            for (int hw = 0; hw < 2; hw++) {
+              const unsigned kw = key_pair(wp[rb][nb][hw]);
+              any |= pk_max_u16(kw, bm1[nb]) ^ bm1[nb];                  // non-zero: a key above bound - 1
+              mag = pk_max_u16(mag, wp[rb][nb][hw] & 0x7FFF7FFFu);       // above 0x7F80: a NaN
+            }
+        const bool look = any != 0u || pk_max_u16(mag, 0x7F807F80u) != 0x7F807F80u;
+        if (__builtin_amdgcn_ballot_w64(look) != 0) {
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int nb = 0; nb < 2; nb++) {
+              const int b = 32 * w + 16 * nb + l16;
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                const int r = 16 * rb + 4 * kg + e;
+                const unsigned key = topk_key((unsigned short)(wp[rb][nb][e >> 1] >> (16 * (e & 1))));
+                if (look && key >= bkey[nb] && r < nvalid && b < p.batch) {
+                  const unsigned long long ent = ((unsigned long long)b << 48) | ((unsigned long long)key << 32) |
+                                                 (unsigned long long)(0xFFFFFFFFu - (unsigned)(label0 + r));
+                  const unsigned qs = atomicAdd(q_cnt, 1u);
+                  if (qs < (unsigned)SEL_QUEUE) q_ent[qs] = ent;
+                  else emit(ent);   // queue full (many logits at the bound): straight to the list
+                }
+              }
+            }
+        }
+      }
+      if (more) asm volatile("s_waitcnt vmcnt(%0)" : : "n"(FWD_DMA) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();   // the next tile has landed for every wavefront, and this one has been read by all
+      buf = buf == 2 ? 0 : buf + 1;
+      if (MODE == 1 && (++since == SEL_FLUSH || j + nblocks >= p.n_visit)) {
+        // Candidates wait in an LDS queue and move to the rows' lists every few tiles: the list slot comes from an
+        // atomic whose result a wavefront has to wait for, together with its outstanding tile loads.  Nobody adds to the
+        // queue between the barrier above and the one below.
+        since = 0;
+        const unsigned qn = *q_cnt < (unsigned)SEL_QUEUE ? *q_cnt : (unsigned)SEL_QUEUE;
+        for (unsigned i = tid; i < qn; i += NT) emit(q_ent[i]);
+        __syncthreads();
+        if (tid == 0) *q_cnt = 0u;
+        __syncthreads();
+      }
+    }
+  }
+  if (MODE == 0) {
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      unsigned m = mx[nb] & 0xFFFFu, h = mx[nb] >> 16;
+      m = m > h ? m : h;
+      const unsigned o1 = __shfl_xor(m, 16, 64);
+      m = m > o1 ? m : o1;
+      const unsigned o2 = __shfl_xor(m, 32, 64);
+      m = m > o2 ? m : o2;
+      if (kg == 0) p.gmax[(size_t)block * BP + 32 * w + 16 * nb + l16] = (unsigned short)m;
+    }
+  }
+}
+
 }  // namespace xmc

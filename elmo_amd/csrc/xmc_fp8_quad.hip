@@ -602,6 +602,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
 #pragma unroll
         for (int cg = 0; cg < 3; cg++) wq[nb][cg] = *(const unsigned*)(lds + wrow + 16 * nbg * QWS + 4 * cg);
       }
+      // all 24 matrix instructions first: the second block's run in the matrix pipe while the first block is updated
+      floatx4 aa[2][3];
+#pragma unroll
+      for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+        for (int cg = 0; cg < 3; cg++) {
+          aa[nb][cg] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < 4; ks++) aa[nb][cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][ks], bg[nb][ks], aa[nb][cg], 0, 0, 0);
+        }
+      QFENCE();
 #pragma unroll
       for (int nb = 0; nb < 2; nb++) {
         const int nbg = 2 * h + nb;
@@ -610,9 +621,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_quad_kernel(const QuadParams 
         float t[3][4];
 #pragma unroll
         for (int cg = 0; cg < 3; cg++) {
-          floatx4 a = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int ks = 0; ks < 4; ks++) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][ks], bg[nb][ks], a, 0, 0, 0);
+          const floatx4 a = aa[nb][cg];
           const unsigned wv = wq[nb][cg];
           floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, true);
           t[cg][0] = __builtin_fmaf(-p.lr_eff, a[0], w01.x); t[cg][1] = __builtin_fmaf(-p.lr_eff, a[1], w01.y);

@@ -25,14 +25,6 @@ typedef TopkBins<1024> B1024;
 constexpr int TOPK_CAP = 6144;  // chunk logits at or above the bound that one workgroup keeps in LDS
 constexpr int TOPK_SMALL = 512; // candidates (kept entries included) that are ranked directly
 
-// ascending key order == ascending value order
-__device__ __forceinline__ unsigned topk_key(unsigned short bits) {
-  return (bits & 0x8000u) ? (unsigned)(~bits & 0xFFFFu) : (unsigned)(bits | 0x8000u);
-}
-__device__ __forceinline__ unsigned short topk_bits(unsigned key) {
-  return (key & 0x8000u) ? (unsigned short)(key & 0x7FFFu) : (unsigned short)(~key & 0xFFFFu);
-}
-
 // z: a row's logits of the chunk at z + row*stride, n_all of them valid (n_all <= 2^17; stride % 4 == 0; z 8-byte aligned)
 // run_val/run_idx: [batch][2][TOPK_MAX] entries kept so far: every batch row has two lists, which topk_finish_kernel
 // merges.  parts = 1: one workgroup per row adds all n_all logits to list 0 (have0 entries valid).  parts = 2: two
@@ -318,6 +310,75 @@ __global__ __launch_bounds__(2 * TOPK_MAX) void topk_finish_kernel(const unsigne
   if (pos < k) {
     out_val[(size_t)b * k + pos] = bits;
     out_idx[(size_t)b * k + pos] = idx;
+  }
+}
+
+
+// ---- the two small kernels of the two-pass top-k (fp8_forward_select_kernel produces gmax and the candidate lists)
+
+// bound[b] = k-th largest of the `groups` maxima gmax[g][b] of batch row b (groups >= k); rows at or past `batch` get
+// a bound nothing reaches.  Also clears the candidate counts and the status word.  One workgroup of TOPK_GROUPS threads
+// per row of the padded batch.
+constexpr int TOPK_GROUPS = 512;
+__global__ __launch_bounds__(TOPK_GROUPS) void topk_bound_kernel(const unsigned short* gmax, int groups, int k, int batch,
+                                                                 unsigned short* bound, unsigned* count, int* status) {
+  __shared__ __attribute__((aligned(16))) unsigned keys[TOPK_GROUPS];
+  const int b = blockIdx.x, g = threadIdx.x;
+  if (g == 0) {
+    count[b] = 0u;
+    if (b == 0) *status = 0;
+    if (b >= batch) bound[b] = 0xFFFFu;
+  }
+  if (b >= batch) return;
+  const unsigned key = g < groups ? (unsigned)gmax[(size_t)g * BP + b] : 0u;
+  keys[g] = key;
+  __syncthreads();
+  if (g >= groups) return;
+  int rank = 0;   // groups before this one in the order key descending, group ascending
+  for (int j = 0; j < TOPK_GROUPS; j += 4) {
+    const uint4 kj = *(const uint4*)(keys + j);
+    rank += (kj.x > key || (kj.x == key && j < g)) ? 1 : 0;
+    rank += (kj.y > key || (kj.y == key && j + 1 < g)) ? 1 : 0;
+    rank += (kj.z > key || (kj.z == key && j + 2 < g)) ? 1 : 0;
+    rank += (kj.w > key || (kj.w == key && j + 3 < g)) ? 1 : 0;
+  }
+  if (rank == k - 1) bound[b] = (unsigned short)key;
+}
+
+// Ranks the candidate list of batch row b (label and key per entry, all labels different) and writes its k largest to the
+// outputs [batch][k]: value descending, label ascending among equal values.  status |= 1 if a row collected more
+// candidates than its list holds (the outputs of that call are then not to be used), |= 2 if a row has fewer than k.
+constexpr int TOPK_LIST = 1024;   // == SEL_CAP of the producing kernel
+__global__ __launch_bounds__(TOPK_LIST) void topk_pick_kernel(const unsigned* cand_label, const unsigned short* cand_key,
+                                                              const unsigned* count, int k, unsigned short* out_val, int* out_idx,
+                                                              int* status) {
+  __shared__ __attribute__((aligned(16))) unsigned long long ent[TOPK_LIST];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const unsigned have = count[b];
+  const int n = have < (unsigned)TOPK_LIST ? (int)have : TOPK_LIST;
+  if (tid == 0 && (have > (unsigned)TOPK_LIST || n < k)) atomicOr(status, have > (unsigned)TOPK_LIST ? 1 : 2);
+  // key << 32 | ~label: larger = better value, then smaller label; 0 ranks after every entry
+  const unsigned long long mine = tid < n ? ((unsigned long long)cand_key[(size_t)b * TOPK_LIST + tid] << 32) |
+                                                (unsigned long long)(0xFFFFFFFFu - cand_label[(size_t)b * TOPK_LIST + tid])
+                                          : 0ull;
+  ent[tid] = mine;
+  __syncthreads();
+  if (tid < n) {
+    int rank = 0;
+    const int n2 = (n + 1) & ~1;
+    for (int j = 0; j < n2; j += 2) {
+      const ulonglong2 e = *(const ulonglong2*)(ent + j);
+      rank += e.x > mine ? 1 : 0;
+      rank += e.y > mine ? 1 : 0;
+    }
+    if (rank < k) {
+      out_val[(size_t)b * k + rank] = topk_bits((unsigned)(mine >> 32));
+      out_idx[(size_t)b * k + rank] = (int)(0xFFFFFFFFu - (unsigned)mine);
+    }
+  }
+  if (tid >= n && tid < k) {   // fewer than k candidates (reported above): -inf, label -1
+    out_val[(size_t)b * k + tid] = 0xFF80;
+    out_idx[(size_t)b * k + tid] = -1;
   }
 }
 

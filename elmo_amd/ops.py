@@ -107,10 +107,21 @@ def topk_scratch_bytes(rows_per_chunk):
     return n
 
 
-def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspace=None, scratch=None):
+def topk_fused_scratch_bytes():
+    return _lib.load().xmc_topk_fused_scratch_bytes()
+
+
+def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspace=None, scratch=None, fused=True,
+                     fused_scratch=None, defer_check=False):
     """values, indices = top-k of the inference logits per row (what evaluate.py:158-159 computes as
     xfc_forward(embed).topk(k)), without the dense [B, num_labels] matrix.  values bf16 [B, k] descending, indices int64
-    [B, k]; equal values are ordered by ascending label id."""
+    [B, k]; equal values are ordered by ascending label id.
+
+    fused=True takes the two-pass kernels (selection inside the logits kernel, < 1 MB of scratch) where the label count
+    allows and reads their status word back: a call that reports an overflowing candidate list (massive ties) is
+    repeated on the general path, as are shapes the fused path does not take.  defer_check=True skips that read-back
+    (no synchronisation) and returns (values, indices, status) with status an int32 device tensor, one word per slice
+    of 128 rows, that the caller has to find zero before using the result."""
     lib = _lib.load()
     assert x.is_cuda and x.dim() == 2 and x.shape[1] == FEATURES
     assert 0 < k <= TOPK_MAX and k <= num_labels, "k must be between 1 and 128"
@@ -119,27 +130,47 @@ def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspa
     nc = len(chunks)
     if workspace is None:
         workspace = alloc_workspace(nc, rows, x.device)
-    need = lib.xmc_topk_scratch_bytes(rows)
-    if scratch is None or scratch.numel() < need:
-        scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
     total = xb.shape[0]
     vals = torch.empty(total, k, dtype=torch.bfloat16, device=x.device)
     idx = torch.empty(total, k, dtype=torch.int32, device=x.device)
-    for lo in range(0, total, MAX_BATCH):
+    nslices = (total + MAX_BATCH - 1) // MAX_BATCH
+    status = torch.zeros(nslices, dtype=torch.int32, device=x.device)
+    for si, lo in enumerate(range(0, total, MAX_BATCH)):
         hi = min(lo + MAX_BATCH, total)
         n = hi - lo
         npad = (n + 15) // 16 * 16
         xs = xb[lo:hi]
         if npad != n:
-            xs = torch.cat([xs, torch.zeros(npad - n, FEATURES, dtype=xb.dtype, device=xb.device)])
+            # rows that pad the batch to a multiple of 16 repeat the last row (rows of zeros would tie on every label
+            # and overflow the two-pass path's candidate lists); their results are dropped below
+            xs = torch.cat([xs, xs[-1:].expand(npad - n, FEATURES)])
         tv = torch.empty(npad, k, dtype=torch.bfloat16, device=x.device)
         ti = torch.empty(npad, k, dtype=torch.int32, device=x.device)
-        st = lib.xmc_fp8_forward_topk(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
-                                      int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
-                                      workspace.numel(), scratch.data_ptr(), scratch.numel(), _stream_ptr())
-        _lib.check(st, "xmc_fp8_forward_topk")
+        done = False
+        if fused:
+            need = lib.xmc_topk_fused_scratch_bytes()
+            if fused_scratch is None or fused_scratch.numel() < need:
+                fused_scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+            st = lib.xmc_fp8_forward_topk_fused(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
+                                                int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
+                                                workspace.numel(), fused_scratch.data_ptr(), fused_scratch.numel(),
+                                                status[si:].data_ptr(), _stream_ptr())
+            if st != _lib.XMC_ERR_RANGE:
+                _lib.check(st, "xmc_fp8_forward_topk_fused")
+                done = defer_check or int(status[si].item()) == 0
+        if not done:
+            need = lib.xmc_topk_scratch_bytes(rows)
+            if scratch is None or scratch.numel() < need:
+                scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+            st = lib.xmc_fp8_forward_topk(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
+                                          int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
+                                          workspace.numel(), scratch.data_ptr(), scratch.numel(), _stream_ptr())
+            _lib.check(st, "xmc_fp8_forward_topk")
+            status[si] = 0
         vals[lo:hi] = tv[:n]
         idx[lo:hi] = ti[:n]
+    if defer_check:
+        return vals, idx.to(torch.int64), status
     return vals, idx.to(torch.int64)
 
 

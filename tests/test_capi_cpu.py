@@ -21,7 +21,7 @@ def test_every_declared_symbol_is_exported():
     lib = _lib.load()
     names = declared_functions()
     assert {"xmc_version", "xmc_error_string", "xmc_workspace_bytes", "xmc_fp8_step", "xmc_fp8_forward",
-            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes"} <= set(names)
+            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes", "xmc_fp8_forward_topk_fused", "xmc_topk_fused_scratch_bytes"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -119,3 +119,23 @@ def test_static_forward_rejects_bad_arguments_before_touching_the_device():
     assert call(batch=144) == -2 and call(batch=8) == -2 and call(feat=1024) == -2 and call(rows=40) == -2
     assert call(nc=65) == -4
     assert call(x=P + 2) == -3
+
+
+def test_two_pass_topk_rejects_bad_arguments_before_touching_the_device():
+    lib = _lib.load()
+    need = lib.xmc_topk_fused_scratch_bytes()
+    assert 0 < need < 1000000                       # group maxima, bounds, counts, 1,024 candidates per row
+    P = 0x7F0000001000
+    arr = (ctypes.c_void_p * 1)(P)
+    wsb = lib.xmc_workspace_bytes(1, 1 << 20)
+
+    def call(**k):
+        return lib.xmc_fp8_forward_topk_fused(k.get("arr", arr), 1, k.get("rows", 1 << 20), P, 16, k.get("feat", 768), 1.0, 1.0,
+                                              k.get("labels", 1 << 20), k.get("k", 100), P, P, P, k.get("wsb", wsb),
+                                              k.get("scratch", P), k.get("sb", need), k.get("status", P), None)
+    assert call(arr=None) == -1 and call(scratch=None) == -1 and call(status=None) == -1
+    assert call(feat=1024) == -2 and call(k=0) == -2 and call(k=129) == -2 and call(labels=(1 << 20) + 1) == -2
+    assert call(scratch=P + 16) == -3 and call(status=P + 2) == -3
+    assert call(sb=need - 1) == -5 and call(wsb=wsb - 1) == -5
+    # too few labels for a bound from sampled tiles: fewer than 4 k tiles of 32 labels
+    assert call(labels=12000, k=100) == -4 and call(labels=600, k=5) == -4

@@ -50,15 +50,17 @@ def test_forward_scales(gpu):
     (3, 16384, 32, 49000, 100),     # one group above 32,768 labels: two workgroups and two lists per batch row
     (5, 16384, 16, 81920, 7),       # the same, k small, nothing dropped
 ])
-def test_topk_forward(gpu, nc, rows, batch, num_labels, k):
-    """Chunk-wise top-k against the dense logits of the same library (bit-equal values, ids that point at them, the
+@pytest.mark.parametrize("fused", [False, True])
+def test_topk_forward(gpu, nc, rows, batch, num_labels, k, fused):
+    """Top-k without the dense logits - the chunk-wise path, and the two-pass path where the label count admits it (the
+    op falls back by itself where it does not) - against the dense logits of the same library (bit-equal values, ids that point at them, the
     documented order among ties) and against the oracle's top-k of the oracle's logits."""
     import torch
     from elmo_amd import ops
     case = H.make_case(nc, rows, batch, 70 + nc, std=0.5)
     chunks, x, _ = H.to_device_case(case, gpu)
     dense = ops.fp8_forward(chunks, x, num_labels).float().cpu().numpy()
-    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k)
+    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=fused)
     assert vals.shape == (batch, k) and idx.shape == (batch, k) and idx.dtype == torch.int64
     v, i = vals.float().cpu().numpy(), idx.cpu().numpy()
     want_v, want_i = O.topk_of_logits(dense, k)
@@ -88,8 +90,9 @@ def test_topk_with_repeated_values(gpu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("k,nc", [(100, 2), (7, 2), (100, 3), (7, 3)])
-def test_topk_when_most_logits_tie(gpu, k, nc):
+def test_topk_when_most_logits_tie(gpu, k, nc, fused):
     """Nearly all rows of W are one and the same row: more logits reach the running bound than the selection keeps in
     fast memory, and the k-th value is a tie of thousands that the label id has to break - with three chunks across
     the two lists of a batch row, which the last kernel merges."""
@@ -105,12 +108,17 @@ def test_topk_when_most_logits_tie(gpu, k, nc):
     chunks, x, _ = H.to_device_case(case, gpu)
     num_labels = nc * rows - 5
     dense = ops.fp8_forward(chunks, x, num_labels).float().cpu().numpy()
-    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k)
+    vals, idx = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=fused)
     want_v, want_i = O.topk_of_logits(dense, k)
     assert np.array_equal(vals.float().cpu().numpy(), want_v) and np.array_equal(idx.cpu().numpy(), want_i)
+    if fused:
+        # the two-pass path by itself reports that a candidate list overflowed (the op above then repeated the call)
+        _, _, status = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=True, defer_check=True)
+        assert int(status[0]) & 1
 
 
-def test_topk_at_the_shipped_670k_geometry(gpu):
+@pytest.mark.parametrize("fused", [False, True])
+def test_topk_at_the_shipped_670k_geometry(gpu, fused):
     """amazontitles670k.yaml ships num_chunks: 2, i.e. chunks of 335,056 rows: larger than one selection segment, so each
     chunk is taken in three pieces.  Against torch.topk of the library's own dense logits (values bit-equal; ids point at
     those values and agree wherever the value is unique in its row)."""
@@ -123,7 +131,11 @@ def test_topk_at_the_shipped_670k_geometry(gpu):
     chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.3).to(torch.float8_e4m3fn) for _ in range(nc)]
     x = torch.from_numpy(synth.make_x(batch, 768, 13)).to(gpu).to(torch.bfloat16)
     dense = ops.fp8_forward(chunks, x, L)
-    vals, idx = ops.fp8_forward_topk(chunks, x, L, k)
+    if fused:
+        vals, idx, status = ops.fp8_forward_topk(chunks, x, L, k, fused=True, defer_check=True)
+        assert int(status[0]) == 0                 # the two-pass path produced this result itself
+    else:
+        vals, idx = ops.fp8_forward_topk(chunks, x, L, k, fused=False)
     tv, ti = torch.topk(dense.float(), k, dim=1)
     assert torch.equal(vals.float(), tv)
     assert torch.equal(dense.float().gather(1, idx), tv) and int(idx.max()) < L and int(idx.min()) >= 0
@@ -135,3 +147,58 @@ def test_topk_at_the_shipped_670k_geometry(gpu):
     assert np.array_equal(i[uniq], ti.cpu().numpy()[uniq])
     # labels from both chunks and from all three pieces of a chunk appear
     assert (i >= rows).any() and (i < rows).any()
+
+
+@pytest.mark.parametrize("k,batch,num_labels", [(100, 128, 262144 - 7), (5, 50, 200000), (128, 16, 140000), (1, 16, 70000)])
+def test_two_pass_topk_equals_the_chunkwise_one(gpu, k, batch, num_labels):
+    """The two selections through the C ABI on the same weights: bit-equal values, equal label ids (both order equal
+    values by ascending label id), status word zero, and the sampled first pass at every stride (k = 1 and 5 visit one
+    tile in 16, k = 100 and 128 one in 4)."""
+    import torch
+    from elmo_amd import ops
+    nc = 4
+    rows = (num_labels + 16 * nc - num_labels % (16 * nc)) // nc
+    gen = torch.Generator(device=gpu).manual_seed(100 + k)
+    chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.4).to(torch.float8_e4m3fn) for _ in range(nc)]
+    x = torch.from_numpy(synth.make_x(batch, 768, 14)).to(gpu).to(torch.bfloat16)
+    v0, i0 = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=False)
+    v1, i1, status = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=True, defer_check=True)
+    assert int(status.abs().sum()) == 0
+    assert torch.equal(v0.view(torch.int16), v1.view(torch.int16)) and torch.equal(i0, i1)
+    # a second call on the same scratch-free path gives the same again (counts and status are reset by the call)
+    v2, i2, status = ops.fp8_forward_topk(chunks, x, num_labels, k, fused=True, defer_check=True)
+    assert int(status.abs().sum()) == 0 and torch.equal(v1.view(torch.int16), v2.view(torch.int16)) and torch.equal(i1, i2)
+
+
+def test_two_pass_topk_with_heads_first_and_nan(gpu):
+    """Labels sorted by frequency put the large logits into the first rows: the first pass samples tiles across the
+    whole range, so its bound stays useful (status zero).  Two weight rows hold a NaN code (0x7F, 0xFF): their logits
+    are NaN, which orders above every number as in torch.topk, whatever its sign, the smaller label first."""
+    import torch
+    from elmo_amd import ops
+    L, nc, k, batch = 160000, 2, 100, 32
+    rows = L // nc
+    gen = torch.Generator(device=gpu).manual_seed(21)
+    scale = torch.linspace(1.5, 0.05, L, device=gpu).unsqueeze(1)       # head labels first
+    w = torch.randn(L, 768, generator=gen, device=gpu) * scale
+    w8 = w.to(torch.float8_e4m3fn)
+    raw = w8.view(torch.uint8)
+    raw[1234, 5] = 0x7F
+    raw[150001, 700] = 0xFF
+    chunks = [w8[c * rows:(c + 1) * rows].contiguous() for c in range(nc)]
+    x = torch.from_numpy(synth.make_x(batch, 768, 15)).to(gpu).to(torch.bfloat16)
+    dense = ops.fp8_forward(chunks, x, L).float()
+    assert torch.isnan(dense[:, 1234]).all() and torch.isnan(dense[:, 150001]).all()
+    for fused in (True, False):
+        if fused:
+            vals, idx, status = ops.fp8_forward_topk(chunks, x, L, k, fused=True, defer_check=True)
+            assert int(status[0]) == 0
+        else:
+            vals, idx = ops.fp8_forward_topk(chunks, x, L, k, fused=False)
+        v = vals.float()
+        assert torch.isnan(v[:, :2]).all() and not torch.isnan(v[:, 2:]).any()
+        assert torch.equal(idx[:, 0], torch.full_like(idx[:, 0], 1234)) and torch.equal(idx[:, 1], torch.full_like(idx[:, 1], 150001))
+        finite = dense.clone()
+        finite[:, 1234] = -float("inf"); finite[:, 150001] = -float("inf")
+        tv, _ = torch.topk(finite, k - 2, dim=1)
+        assert torch.equal(v[:, 2:], tv) and torch.equal(dense.gather(1, idx[:, 2:]), tv)
