@@ -68,7 +68,7 @@ def load():
     lib.xmc_topk_fused_scratch_bytes.argtypes = []
     lib.xmc_fp8_forward_topk_fused.restype = i32
     lib.xmc_fp8_forward_topk_fused.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp,
-                                               vp, vp, sz, vp, sz, vp, vp]
+                                               vp, i32, vp, sz, vp, sz, vp, vp]
     lib.xmc_step_error_offset.restype = sz
     lib.xmc_step_workgroups.restype = i32
     lib.xmc_step_xcc_ids.restype = i32

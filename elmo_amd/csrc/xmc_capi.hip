@@ -379,12 +379,12 @@ static int topk_fused_step(int tiles, int k) {
 
 int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
                                int features, float scale_w, float scale_x, long long num_labels, int k, void* out_val_bf16,
-                               int32_t* out_idx, void* workspace, size_t workspace_bytes, void* scratch, size_t scratch_bytes,
-                               int32_t* status, void* stream_) {
+                               void* out_idx, int idx_int64, void* workspace, size_t workspace_bytes, void* scratch,
+                               size_t scratch_bytes, int32_t* status, void* stream_) {
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
   if (!out_val_bf16 || !out_idx || !scratch || !status) return XMC_ERR_NULL;
-  if (((uintptr_t)scratch & 255) != 0 || ((uintptr_t)status & 3) != 0) return XMC_ERR_ALIGN;
+  if (((uintptr_t)scratch & 255) != 0 || ((uintptr_t)status & 3) != 0 || ((uintptr_t)out_idx & (idx_int64 ? 7 : 3)) != 0) return XMC_ERR_ALIGN;
   if (scratch_bytes < SELS_BYTES) return XMC_ERR_WORKSPACE;
   if (num_labels <= 0 || num_labels > (long long)num_chunks * rows_per_chunk) return XMC_ERR_SHAPE;
   if (k <= 0 || k > TOPK_MAX || k > num_labels) return XMC_ERR_SHAPE;
@@ -423,7 +423,8 @@ int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows
   sp.tile_step = 1;
   sp.n_visit = tiles;
   fp8_forward_select_kernel<1><<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, SEL_LDS, stream>>>(sp);
-  topk_pick_kernel<<<batch, TOPK_LIST, 0, stream>>>(sp.cand_label, sp.cand_key, sp.count, k, (unsigned short*)out_val_bf16, out_idx, status);
+  topk_pick_kernel<<<batch, TOPK_LIST, 0, stream>>>(sp.cand_label, sp.cand_key, sp.count, k, (unsigned short*)out_val_bf16, out_idx,
+                                                    idx_int64 ? 1 : 0, status);
   return launch_status();
 }
 

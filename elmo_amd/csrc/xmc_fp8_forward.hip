@@ -240,9 +240,10 @@ __device__ __forceinline__ unsigned pk_max_u16(unsigned a, unsigned b) {
   return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(ushortx2, a), __builtin_bit_cast(ushortx2, b)));
 }
 // order keys of two packed bf16 values (topk_key per half, without its NaN rule: a NaN with the sign bit set gets a small key)
+typedef short shortx2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned key_pair(unsigned w) {
-  const unsigned s = (w >> 15) & 0x00010001u;
-  return w ^ (((s << 16) - s) | 0x80008000u);   // (s << 16) - s: 0xFFFF in the halves whose sign bit is set
+  const unsigned neg = __builtin_bit_cast(unsigned, __builtin_bit_cast(shortx2, w) >> 15);   // 0xFFFF in the negative halves
+  return w ^ (neg | 0x80008000u);
 }
 
 template <int MODE>
@@ -330,8 +331,9 @@ __global__ __launch_bounds__(NT) void fp8_forward_select_kernel(const SelectPara
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
-          wp[rb][nb][0] = bf16_pack2(z[rb][nb][0] * p.zscale, z[rb][nb][1] * p.zscale);
-          wp[rb][nb][1] = bf16_pack2(z[rb][nb][2] * p.zscale, z[rb][nb][3] * p.zscale);
+          if (p.zscale != 1.0f) z[rb][nb] *= p.zscale;   // the same product as the dense kernel's
+          wp[rb][nb][0] = bf16_pack2(z[rb][nb][0], z[rb][nb][1]);
+          wp[rb][nb][1] = bf16_pack2(z[rb][nb][2], z[rb][nb][3]);
         }
       if (MODE == 0) {
 #pragma unroll
@@ -348,36 +350,40 @@ __global__ __launch_bounds__(NT) void fp8_forward_select_kernel(const SelectPara
               mx[nb] = pk_max_u16(mx[nb], kw);
             }
       } else {
-        unsigned any = 0u, mag = 0u;
+        unsigned hit[2][2][2], any = 0u, top = 0u;
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll
           for (int nb = 0; nb < 2; nb++)
 #pragma unroll
             for (int hw = 0; hw < 2; hw++) {
-              const unsigned kw = key_pair(wp[rb][nb][hw]);
-              any |= pk_max_u16(kw, bm1[nb]) ^ bm1[nb];                  // non-zero: a key above bound - 1
-              mag = pk_max_u16(mag, wp[rb][nb][hw] & 0x7FFF7FFFu);       // above 0x7F80: a NaN
+              hit[rb][nb][hw] = pk_max_u16(key_pair(wp[rb][nb][hw]), bm1[nb]) ^ bm1[nb];   // non-zero: a key above bound - 1
+              any |= hit[rb][nb][hw];
+              top = pk_max_u16(top, wp[rb][nb][hw]);                                      // a half above 0xFF80: a NaN with the sign bit
             }
-        const bool look = any != 0u || pk_max_u16(mag, 0x7F807F80u) != 0x7F807F80u;
-        if (__builtin_amdgcn_ballot_w64(look) != 0) {
+        const bool nan = pk_max_u16(top, 0xFF80FF80u) != 0xFF80FF80u;   // (a NaN without it has a key above every bound)
+        if (__builtin_amdgcn_ballot_w64(any != 0u || nan) != 0) {
 #pragma unroll
           for (int rb = 0; rb < 2; rb++)
 #pragma unroll
             for (int nb = 0; nb < 2; nb++) {
               const int b = 32 * w + 16 * nb + l16;
 #pragma unroll
-              for (int e = 0; e < 4; e++) {
-                const int r = 16 * rb + 4 * kg + e;
-                const unsigned key = topk_key((unsigned short)(wp[rb][nb][e >> 1] >> (16 * (e & 1))));
-                if (look && key >= bkey[nb] && r < nvalid && b < p.batch) {
-                  const unsigned long long ent = ((unsigned long long)b << 48) | ((unsigned long long)key << 32) |
-                                                 (unsigned long long)(0xFFFFFFFFu - (unsigned)(label0 + r));
-                  const unsigned qs = atomicAdd(q_cnt, 1u);
-                  if (qs < (unsigned)SEL_QUEUE) q_ent[qs] = ent;
-                  else emit(ent);   // queue full (many logits at the bound): straight to the list
+              for (int hw = 0; hw < 2; hw++)
+                if ((hit[rb][nb][hw] != 0u || nan) && b < p.batch) {
+#pragma unroll
+                  for (int e = 0; e < 2; e++) {
+                    const int r = 16 * rb + 4 * kg + 2 * hw + e;
+                    const unsigned key = topk_key((unsigned short)(wp[rb][nb][hw] >> (16 * e)));
+                    if (key >= bkey[nb] && r < nvalid) {
+                      const unsigned long long ent = ((unsigned long long)b << 48) | ((unsigned long long)key << 32) |
+                                                     (unsigned long long)(0xFFFFFFFFu - (unsigned)(label0 + r));
+                      const unsigned qs = atomicAdd(q_cnt, 1u);
+                      if (qs < (unsigned)SEL_QUEUE) q_ent[qs] = ent;
+                      else emit(ent);   // queue full (many logits at the bound): straight to the list
+                    }
+                  }
                 }
-              }
             }
         }
       }

@@ -316,13 +316,35 @@ __global__ __launch_bounds__(2 * TOPK_MAX) void topk_finish_kernel(const unsigne
 
 // ---- the two small kernels of the two-pass top-k (fp8_forward_select_kernel produces gmax and the candidate lists)
 
+// The k-th largest of the 16-bit keys that the threads of a workgroup hold (one per thread; `valid` false = no key), or
+// 0 if fewer than k are valid: the largest T with at least k keys >= T, found bit by bit from the top.  Every thread of
+// the workgroup calls this; wcnt = 2 x WAVES words of LDS.
+template <int WAVES>
+__device__ __forceinline__ unsigned block_kth_key(unsigned key, bool valid, int k, unsigned* wcnt) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  unsigned T = 0u;
+#pragma unroll 1
+  for (int bit = 15; bit >= 0; bit--) {
+    const unsigned c = T | (1u << bit);
+    const unsigned long long m = __ballot(valid && key >= c);
+    unsigned* mine = wcnt + ((bit & 1) ? WAVES : 0);   // alternating halves: a slow reader is never overtaken by a writer
+    if (lane == 0) mine[wave] = (unsigned)__popcll(m);
+    __syncthreads();
+    unsigned total = 0;
+#pragma unroll
+    for (int q = 0; q < WAVES; q++) total += mine[q];
+    if (total >= (unsigned)k) T = c;
+  }
+  return T;
+}
+
 // bound[b] = k-th largest of the `groups` maxima gmax[g][b] of batch row b (groups >= k); rows at or past `batch` get
 // a bound nothing reaches.  Also clears the candidate counts and the status word.  One workgroup of TOPK_GROUPS threads
 // per row of the padded batch.
 constexpr int TOPK_GROUPS = 512;
 __global__ __launch_bounds__(TOPK_GROUPS) void topk_bound_kernel(const unsigned short* gmax, int groups, int k, int batch,
                                                                  unsigned short* bound, unsigned* count, int* status) {
-  __shared__ __attribute__((aligned(16))) unsigned keys[TOPK_GROUPS];
+  __shared__ unsigned wcnt[2 * (TOPK_GROUPS / 64)];
   const int b = blockIdx.x, g = threadIdx.x;
   if (g == 0) {
     count[b] = 0u;
@@ -331,54 +353,65 @@ __global__ __launch_bounds__(TOPK_GROUPS) void topk_bound_kernel(const unsigned 
   }
   if (b >= batch) return;
   const unsigned key = g < groups ? (unsigned)gmax[(size_t)g * BP + b] : 0u;
-  keys[g] = key;
-  __syncthreads();
-  if (g >= groups) return;
-  int rank = 0;   // groups before this one in the order key descending, group ascending
-  for (int j = 0; j < TOPK_GROUPS; j += 4) {
-    const uint4 kj = *(const uint4*)(keys + j);
-    rank += (kj.x > key || (kj.x == key && j < g)) ? 1 : 0;
-    rank += (kj.y > key || (kj.y == key && j + 1 < g)) ? 1 : 0;
-    rank += (kj.z > key || (kj.z == key && j + 2 < g)) ? 1 : 0;
-    rank += (kj.w > key || (kj.w == key && j + 3 < g)) ? 1 : 0;
-  }
-  if (rank == k - 1) bound[b] = (unsigned short)key;
+  const unsigned T = block_kth_key<TOPK_GROUPS / 64>(key, g < groups, k, wcnt);
+  if (g == 0) bound[b] = (unsigned short)T;
 }
 
-// Ranks the candidate list of batch row b (label and key per entry, all labels different) and writes its k largest to the
-// outputs [batch][k]: value descending, label ascending among equal values.  status |= 1 if a row collected more
-// candidates than its list holds (the outputs of that call are then not to be used), |= 2 if a row has fewer than k.
+// Picks the k best of the candidate list of batch row b (label and key per entry, all labels different) and writes
+// them to the outputs [batch][k]: value descending, label ascending among equal values; labels as int32 or, with
+// idx64, as int64.  The k-th largest key T is found first; the entries at or above it (k plus the ties at T) are then
+// ranked against each other, several threads sharing the comparisons of one entry.  status |= 1 if a row collected
+// more candidates than its list holds (the outputs of that call are then not to be used), |= 2 if a row has fewer than k.
 constexpr int TOPK_LIST = 1024;   // == SEL_CAP of the producing kernel
 __global__ __launch_bounds__(TOPK_LIST) void topk_pick_kernel(const unsigned* cand_label, const unsigned short* cand_key,
-                                                              const unsigned* count, int k, unsigned short* out_val, int* out_idx,
-                                                              int* status) {
+                                                              const unsigned* count, int k, unsigned short* out_val, void* out_idx,
+                                                              int idx64, int* status) {
   __shared__ __attribute__((aligned(16))) unsigned long long ent[TOPK_LIST];
+  __shared__ unsigned rank[TOPK_LIST];
+  __shared__ unsigned wcnt[2 * (TOPK_LIST / 64)];
+  __shared__ unsigned s_m;
   const int b = blockIdx.x, tid = threadIdx.x;
   const unsigned have = count[b];
   const int n = have < (unsigned)TOPK_LIST ? (int)have : TOPK_LIST;
-  if (tid == 0 && (have > (unsigned)TOPK_LIST || n < k)) atomicOr(status, have > (unsigned)TOPK_LIST ? 1 : 2);
-  // key << 32 | ~label: larger = better value, then smaller label; 0 ranks after every entry
-  const unsigned long long mine = tid < n ? ((unsigned long long)cand_key[(size_t)b * TOPK_LIST + tid] << 32) |
-                                                (unsigned long long)(0xFFFFFFFFu - cand_label[(size_t)b * TOPK_LIST + tid])
-                                          : 0ull;
-  ent[tid] = mine;
+  if (tid == 0) {
+    if (have > (unsigned)TOPK_LIST || n < k) atomicOr(status, have > (unsigned)TOPK_LIST ? 1 : 2);
+    s_m = 0u;
+  }
+  rank[tid] = 0u;
+  const unsigned key = tid < n ? (unsigned)cand_key[(size_t)b * TOPK_LIST + tid] : 0u;
+  const unsigned label = tid < n ? cand_label[(size_t)b * TOPK_LIST + tid] : 0u;
+  const unsigned T = block_kth_key<TOPK_LIST / 64>(key, tid < n, k, wcnt);   // its barriers also publish s_m and rank
+  if (tid < n && key >= T) {
+    // key << 32 | ~label: larger = better value, then smaller label
+    ent[atomicAdd(&s_m, 1u)] = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - label);
+  }
   __syncthreads();
-  if (tid < n) {
-    int rank = 0;
-    const int n2 = (n + 1) & ~1;
-    for (int j = 0; j < n2; j += 2) {
-      const ulonglong2 e = *(const ulonglong2*)(ent + j);
-      rank += e.x > mine ? 1 : 0;
-      rank += e.y > mine ? 1 : 0;
-    }
-    if (rank < k) {
-      out_val[(size_t)b * k + rank] = topk_bits((unsigned)(mine >> 32));
-      out_idx[(size_t)b * k + rank] = (int)(0xFFFFFFFFu - (unsigned)mine);
+  const int m = (int)s_m;                       // >= min(k, n) entries, all different
+  int mp = 64;
+  while (mp < m) mp <<= 1;                      // threads per slice; TOPK_LIST / mp slices share an entry's comparisons
+  const int slices = TOPK_LIST / mp, i = tid & (mp - 1), sl = tid / mp;
+  const int per = (m + slices - 1) / slices, j0 = sl * per, j1 = j0 + per < m ? j0 + per : m;
+  if (i < m) {
+    const unsigned long long mine = ent[i];
+    unsigned r = 0;
+    for (int j = j0; j < j1; j++) r += ent[j] > mine ? 1u : 0u;
+    if (r != 0u) atomicAdd(&rank[i], r);
+  }
+  __syncthreads();
+  if (tid < m) {
+    const unsigned r = rank[tid];
+    if (r < (unsigned)k) {
+      const unsigned long long mine = ent[tid];
+      const int lab = (int)(0xFFFFFFFFu - (unsigned)mine);
+      out_val[(size_t)b * k + r] = topk_bits((unsigned)(mine >> 32));
+      if (idx64) ((long long*)out_idx)[(size_t)b * k + r] = lab;
+      else ((int*)out_idx)[(size_t)b * k + r] = lab;
     }
   }
-  if (tid >= n && tid < k) {   // fewer than k candidates (reported above): -inf, label -1
+  if (tid >= m && tid < k) {   // fewer than k candidates (reported above): -inf, label -1
     out_val[(size_t)b * k + tid] = 0xFF80;
-    out_idx[(size_t)b * k + tid] = -1;
+    if (idx64) ((long long*)out_idx)[(size_t)b * k + tid] = -1;
+    else ((int*)out_idx)[(size_t)b * k + tid] = -1;
   }
 }
 

@@ -132,9 +132,9 @@ def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspa
         workspace = alloc_workspace(nc, rows, x.device)
     total = xb.shape[0]
     vals = torch.empty(total, k, dtype=torch.bfloat16, device=x.device)
-    idx = torch.empty(total, k, dtype=torch.int32, device=x.device)
+    idx = torch.empty(total, k, dtype=torch.int64, device=x.device)
     nslices = (total + MAX_BATCH - 1) // MAX_BATCH
-    status = torch.zeros(nslices, dtype=torch.int32, device=x.device)
+    status = torch.empty(nslices, dtype=torch.int32, device=x.device)      # every word is written below
     for si, lo in enumerate(range(0, total, MAX_BATCH)):
         hi = min(lo + MAX_BATCH, total)
         n = hi - lo
@@ -144,34 +144,40 @@ def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspa
             # rows that pad the batch to a multiple of 16 repeat the last row (rows of zeros would tie on every label
             # and overflow the two-pass path's candidate lists); their results are dropped below
             xs = torch.cat([xs, xs[-1:].expand(npad - n, FEATURES)])
-        tv = torch.empty(npad, k, dtype=torch.bfloat16, device=x.device)
-        ti = torch.empty(npad, k, dtype=torch.int32, device=x.device)
+            tv = torch.empty(npad, k, dtype=torch.bfloat16, device=x.device)
+        else:
+            tv = vals[lo:hi]                                               # written in place
         done = False
         if fused:
             need = lib.xmc_topk_fused_scratch_bytes()
             if fused_scratch is None or fused_scratch.numel() < need:
                 fused_scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+            ti = idx[lo:hi] if npad == n else torch.empty(npad, k, dtype=torch.int64, device=x.device)
             st = lib.xmc_fp8_forward_topk_fused(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
-                                                int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
+                                                int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), 1, workspace.data_ptr(),
                                                 workspace.numel(), fused_scratch.data_ptr(), fused_scratch.numel(),
                                                 status[si:].data_ptr(), _stream_ptr())
             if st != _lib.XMC_ERR_RANGE:
                 _lib.check(st, "xmc_fp8_forward_topk_fused")
                 done = defer_check or int(status[si].item()) == 0
+                if done and npad != n:
+                    idx[lo:hi] = ti[:n]
         if not done:
             need = lib.xmc_topk_scratch_bytes(rows)
             if scratch is None or scratch.numel() < need:
                 scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+            ti = torch.empty(npad, k, dtype=torch.int32, device=x.device)
             st = lib.xmc_fp8_forward_topk(arr, nc, rows, xs.data_ptr(), npad, FEATURES, float(scale_w), float(scale_x),
                                           int(num_labels), int(k), tv.data_ptr(), ti.data_ptr(), workspace.data_ptr(),
                                           workspace.numel(), scratch.data_ptr(), scratch.numel(), _stream_ptr())
             _lib.check(st, "xmc_fp8_forward_topk")
             status[si] = 0
-        vals[lo:hi] = tv[:n]
-        idx[lo:hi] = ti[:n]
+            idx[lo:hi] = ti[:n]
+        if npad != n:
+            vals[lo:hi] = tv[:n]
     if defer_check:
-        return vals, idx.to(torch.int64), status
-    return vals, idx.to(torch.int64)
+        return vals, idx, status
+    return vals, idx
 
 
 WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}

@@ -122,6 +122,7 @@ size_t xmc_topk_fused_scratch_bytes(void);
  * selection inside the logits kernel: no logits reach memory.  Two passes over the weights: the first visits one tile
  * in 4..16 and yields, per batch row, a lower bound of the k-th largest logit; the second visits every tile and keeps
  * the logits at or above the bound (a few hundred per row), which a last kernel ranks.
+ *   out_idx  device [batch, k] label ids, int32, or int64 (what torch.topk returns) with idx_int64 != 0
  *   status   device int32, written by the call's kernels: 0 = outputs valid; bit 0 = a row had more than 1,024 logits
  *            at or above its bound (massive ties, e.g. constant logits): the outputs of this call are then not to be
  *            used, and xmc_fp8_forward_topk gives the result; bit 1 = a row found fewer than k (not expected).
@@ -131,8 +132,8 @@ size_t xmc_topk_fused_scratch_bytes(void);
  */
 int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
                                int features, float scale_w, float scale_x, long long num_labels, int k, void* out_val_bf16,
-                               int32_t* out_idx, void* workspace, size_t workspace_bytes, void* scratch, size_t scratch_bytes,
-                               int32_t* status, void* stream);
+                               void* out_idx, int idx_int64, void* workspace, size_t workspace_bytes, void* scratch,
+                               size_t scratch_bytes, int32_t* status, void* stream);
 
 /* Benchmarking aid (no counterpart in the reference): the next xmc_fp8_step call records these two HIP events
  * (hipEvent_t, created by the caller) immediately before and after its fused step kernel, on the call's stream,

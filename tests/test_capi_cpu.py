@@ -131,11 +131,12 @@ def test_two_pass_topk_rejects_bad_arguments_before_touching_the_device():
 
     def call(**k):
         return lib.xmc_fp8_forward_topk_fused(k.get("arr", arr), 1, k.get("rows", 1 << 20), P, 16, k.get("feat", 768), 1.0, 1.0,
-                                              k.get("labels", 1 << 20), k.get("k", 100), P, P, P, k.get("wsb", wsb),
+                                              k.get("labels", 1 << 20), k.get("k", 100), P, k.get("idx", P), k.get("i64", 0), P, k.get("wsb", wsb),
                                               k.get("scratch", P), k.get("sb", need), k.get("status", P), None)
     assert call(arr=None) == -1 and call(scratch=None) == -1 and call(status=None) == -1
     assert call(feat=1024) == -2 and call(k=0) == -2 and call(k=129) == -2 and call(labels=(1 << 20) + 1) == -2
     assert call(scratch=P + 16) == -3 and call(status=P + 2) == -3
+    assert call(idx=P + 4, i64=1) == -3 and call(idx=P + 4, i64=0) != -3 and call(idx=P + 2) == -3
     assert call(sb=need - 1) == -5 and call(wsb=wsb - 1) == -5
     # too few labels for a bound from sampled tiles: fewer than 4 k tiles of 32 labels
     assert call(labels=12000, k=100) == -4 and call(labels=600, k=5) == -4
