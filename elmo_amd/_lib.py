@@ -69,6 +69,8 @@ def load():
     lib.xmc_fp8_forward_topk_fused.restype = i32
     lib.xmc_fp8_forward_topk_fused.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, ctypes.c_longlong, i32, vp,
                                                vp, i32, vp, sz, vp, sz, vp, vp]
+    lib.xmc_dropout_quantize.restype = i32
+    lib.xmc_dropout_quantize.argtypes = [vp, i32, i32, i32, f32, ctypes.c_ulonglong, vp, vp]
     lib.xmc_step_error_offset.restype = sz
     lib.xmc_step_workgroups.restype = i32
     lib.xmc_step_xcc_ids.restype = i32

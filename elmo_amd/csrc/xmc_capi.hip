@@ -5,6 +5,7 @@
 #include "xmc_fp8_quad.hip"
 #include "xmc_tiled.hip"
 #include "xmc_topk.hip"
+#include "xmc_dropout.hip"
 #include <stdlib.h>
 
 using namespace xmc;
@@ -425,6 +426,21 @@ int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows
   fp8_forward_select_kernel<1><<<tiles < 2 * di.cus ? tiles : 2 * di.cus, NT, SEL_LDS, stream>>>(sp);
   topk_pick_kernel<<<batch, TOPK_LIST, 0, stream>>>(sp.cand_label, sp.cand_key, sp.count, k, (unsigned short*)out_val_bf16, out_idx,
                                                     idx_int64 ? 1 : 0, status);
+  return launch_status();
+}
+
+int xmc_dropout_quantize(const void* x, int x_type, int rows, int cols, float p, unsigned long long seed, void* out_e4m3,
+                         void* stream_) {
+  if (!x || !out_e4m3) return XMC_ERR_NULL;
+  if (x_type != 0 && x_type != 1) return XMC_ERR_MODE;
+  if (rows <= 0 || cols <= 0 || cols % 4 != 0 || !(p >= 0.f) || !(p < 1.f)) return XMC_ERR_SHAPE;
+  if ((long long)rows * cols > 0x7FFFFFFFll) return XMC_ERR_RANGE;   // the random offsets are 32-bit element indices
+  if (((uintptr_t)x & (x_type == 0 ? 7 : 3)) != 0 || ((uintptr_t)out_e4m3 & 3) != 0) return XMC_ERR_ALIGN;
+  DeviceInfo di = device_info();
+  if (di.ok != 1) return XMC_ERR_DEVICE;
+  const long long n4 = (long long)rows * cols / 4;
+  dropout_quantize_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, (hipStream_t)stream_>>>(x, x_type, n4, cols, p, (unsigned)(seed & 0xFFFFFFFFull),
+                                                                                        (unsigned)(seed >> 32), (unsigned*)out_e4m3);
   return launch_status();
 }
 

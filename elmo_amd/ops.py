@@ -180,6 +180,20 @@ def fp8_forward_topk(chunks, x, num_labels, k, scale_w=1.0, scale_x=1.0, workspa
     return vals, idx
 
 
+def dropout_quantize(x, p, seed):
+    """e4m3 tensor of dropout(x) with Triton's random stream: the reference's prototype of dropout inside the FP8 GEMM's
+    operand load (tma_gemm.py:7-13,34-38) as one pass over the embedding.  x: [M, K] bf16 or float8_e4m3fn, contiguous,
+    K a multiple of 4; element (m, k) is kept when tl.rand(seed, m * K + k) > p and scaled by 1 / (1 - p)."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dim() == 2 and x.is_contiguous()
+    assert x.dtype in (torch.bfloat16, torch.float8_e4m3fn)
+    out = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    st = lib.xmc_dropout_quantize(x.data_ptr(), 0 if x.dtype == torch.bfloat16 else 1, x.shape[0], x.shape[1], float(p),
+                                  int(seed), out.data_ptr(), _stream_ptr())
+    _lib.check(st, "xmc_dropout_quantize")
+    return out
+
+
 WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}
 
 

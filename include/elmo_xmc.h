@@ -135,6 +135,16 @@ int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows
                                void* out_idx, int idx_int64, void* workspace, size_t workspace_bytes, void* scratch,
                                size_t scratch_bytes, int32_t* status, void* stream);
 
+/* Dropout fused with the cast to e4m3 (the reference's prototype `_dropout` on the FP8 GEMM's A operand,
+ * src/triton_kernels/tma_gemm.py:7-13,34-38): out[m][k] = e4m3(keep ? x[m][k] / (1 - p) : 0), keep = tl.rand(seed,
+ * m * cols + k) > p (Philox-4x32-10 word 0 of counter (offset, 0, 0, 0), key = seed, as Triton's uniform fp32), the cast
+ * saturating at +-448.
+ *   x        device [rows, cols] contiguous, bf16 (x_type 0) or e4m3 (x_type 1, what the prototype takes); cols % 4 == 0
+ *   p        drop probability, 0 <= p < 1;  out_e4m3: device [rows, cols] bytes;  rows * cols < 2^31
+ */
+int xmc_dropout_quantize(const void* x, int x_type, int rows, int cols, float p, unsigned long long seed, void* out_e4m3,
+                         void* stream);
+
 /* Benchmarking aid (no counterpart in the reference): the next xmc_fp8_step call records these two HIP events
  * (hipEvent_t, created by the caller) immediately before and after its fused step kernel, on the call's stream,
  * then forgets them.  Pass nulls to cancel. */

@@ -157,6 +157,30 @@ def tl_randint(seed, offsets):
     return philox4x32(offs, z, z, z, seed & 0xFFFFFFFF, seed >> 32)[0]
 
 
+def tl_rand(seed, offsets):
+    """`tl.rand(seed, offs)`: the first Philox word as a uniform fp32 in [0, 1) - the word reinterpreted as int32,
+    negative values mapped to -x - 1, converted to fp32 (nearest even) and multiplied by 4.6566127342e-10 in fp32
+    (Triton language/random.py, uint_to_uniform_float; what the reference's dropout prototype compares with p,
+    tma_gemm.py:8-10).  Pinned by vectors from the Triton library's interpreter in tests/golden/triton_rand.json."""
+    x = tl_randint(seed, offsets).view(np.int32).astype(np.int64)
+    x = np.where(x < 0, -x - 1, x)
+    return (x.astype(np.float32) * np.float32(4.6566127342e-10)).astype(np.float32)
+
+
+def dropout_quantize(x, p, seed, row_stride=None):
+    """e4m3 codes of dropout(x): element (m, k) is kept when tl_rand(seed, m * row_stride + k) > p and then scaled by
+    1 / (1 - p) in fp32, else zero; cast to e4m3 (nearest even, saturating) - `_dropout` of tma_gemm.py:7-13 applied
+    to the whole operand (the prototype calls it per tile with these offsets, tma_gemm.py:34-38).  x: fp32 array [M, K]
+    of bf16 or e4m3 values."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    stride = k if row_stride is None else int(row_stride)
+    offs = (np.arange(m, dtype=np.int64)[:, None] * stride + np.arange(k, dtype=np.int64)[None, :])
+    keep = tl_rand(seed, offs) > np.float32(p)
+    scaled = (x / (np.float32(1.0) - np.float32(p))).astype(np.float32)
+    return e4m3_encode(np.where(keep, scaled, np.float32(0.0)), saturate=True)
+
+
 # --------------------------------------------------------------------------- stochastic rounding
 def sr_add_mask(t, rand, k):
     """The reference bit recipe: add the low k random bits to the fp32 bit pattern, clear the low k bits.

@@ -21,7 +21,7 @@ def test_every_declared_symbol_is_exported():
     lib = _lib.load()
     names = declared_functions()
     assert {"xmc_version", "xmc_error_string", "xmc_workspace_bytes", "xmc_fp8_step", "xmc_fp8_forward",
-            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes", "xmc_fp8_forward_topk_fused", "xmc_topk_fused_scratch_bytes"} <= set(names)
+            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes", "xmc_fp8_forward_topk_fused", "xmc_topk_fused_scratch_bytes", "xmc_dropout_quantize"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -140,3 +140,15 @@ def test_two_pass_topk_rejects_bad_arguments_before_touching_the_device():
     assert call(sb=need - 1) == -5 and call(wsb=wsb - 1) == -5
     # too few labels for a bound from sampled tiles: fewer than 4 k tiles of 32 labels
     assert call(labels=12000, k=100) == -4 and call(labels=600, k=5) == -4
+
+
+def test_dropout_quantize_rejects_bad_arguments_before_touching_the_device():
+    lib = _lib.load()
+    P = 0x7F0000001000
+    call = lambda **k: lib.xmc_dropout_quantize(k.get("x", P), k.get("t", 0), k.get("rows", 16), k.get("cols", 768), k.get("p", 0.1), 40,
+                                                k.get("out", P), None)
+    assert call(x=None) == -1 and call(out=None) == -1
+    assert call(t=2) == -6
+    assert call(cols=770) == -2 and call(rows=0) == -2 and call(p=1.0) == -2 and call(p=-0.1) == -2
+    assert call(rows=1 << 22, cols=1024) == -4
+    assert call(x=P + 4) == -3 and call(x=P + 4, t=1) != -3 and call(out=P + 2) == -3

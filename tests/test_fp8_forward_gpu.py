@@ -202,3 +202,24 @@ def test_two_pass_topk_with_heads_first_and_nan(gpu):
         finite[:, 1234] = -float("inf"); finite[:, 150001] = -float("inf")
         tv, _ = torch.topk(finite, k - 2, dim=1)
         assert torch.equal(v[:, 2:], tv) and torch.equal(dense.gather(1, idx[:, 2:]), tv)
+
+
+@pytest.mark.parametrize("rows,cols,p,seed,as_e4m3", [(128, 768, 0.1, 40, False), (16, 768, 0.7, 123456789012, False),
+                                                       (33, 1024, 0.3, 7, True), (128, 768, 0.0, 1, True)])
+def test_dropout_quantize_matches_the_oracle(gpu, rows, cols, p, seed, as_e4m3):
+    """Dropout fused with the e4m3 cast (the reference's prototype, tma_gemm.py:7-13,34-38) against the oracle: bit-equal
+    codes for bf16 and e4m3 input, a 64-bit seed, p = 0."""
+    import torch
+    from elmo_amd import ops
+    rng = np.random.default_rng(seed % 1000)
+    x = C.bf16_round(rng.standard_normal((rows, cols)).astype(np.float32) * 4.0)
+    x[0, :8] = [500.0, -500.0, 448.0, 0.0, -0.0, 2.0 ** -9, 2.0 ** -10, 300.0]     # saturation, zeros, the smallest codes
+    xd = torch.from_numpy(x).to(gpu).to(torch.bfloat16)
+    if as_e4m3:
+        xd = xd.clamp(-448, 448).to(torch.float8_e4m3fn)         # torch's own cast turns 500 into NaN
+        x = xd.float().cpu().numpy()
+    out = ops.dropout_quantize(xd, p, seed)
+    assert out.dtype == torch.float8_e4m3fn and out.shape == (rows, cols)
+    want = C.dropout_quantize(x, p, seed)
+    got = out.view(torch.uint8).cpu().numpy()
+    assert np.array_equal(got, want)

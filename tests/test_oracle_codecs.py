@@ -88,6 +88,40 @@ def test_tl_randint_recorded_words():
     assert list(C.tl_randint(1024, np.arange(4))) == [3876201247, 854061192, 798737492, 713463838]
 
 
+def test_tl_rand_matches_the_triton_library():
+    """The uniform fp32 of tl.rand against vectors the Triton library in this image produced through its interpreter
+    (tests/golden/make_triton_rand.py): bit-equal, three seeds and offset ranges."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "triton_rand.json")) as f:
+        cases = json.load(f)["cases"]
+    assert len(cases) == 3
+    for key, want in cases.items():
+        seed, start = (int(v) for v in key.split(":"))
+        got = C.tl_rand(seed, np.arange(start, start + len(want))).view(np.uint32)
+        assert np.array_equal(got, np.array(want, dtype=np.uint32)), key
+
+
+def test_dropout_quantize_against_torch_and_its_invariants():
+    """The oracle's dropout + e4m3 cast: kept entries equal torch's CPU cast of x / (1 - p) (a different implementation of
+    the cast), dropped ones are zero, the kept fraction is 1 - p, p = 0 is the plain cast, and the mask depends on
+    (seed, flat offset) only."""
+    rng = np.random.default_rng(5)
+    x = C.bf16_round(rng.standard_normal((64, 768)).astype(np.float32) * 3.0)
+    p, seed = 0.3, 40
+    codes = C.dropout_quantize(x, p, seed)
+    keep = C.tl_rand(seed, np.arange(64 * 768).reshape(64, 768)) > np.float32(p)
+    want = (torch.from_numpy(x) / (1.0 - torch.tensor(p, dtype=torch.float32))).clamp(-448, 448).to(torch.float8_e4m3fn)
+    want = want.view(torch.uint8).numpy()
+    assert np.array_equal(codes[keep], want[keep]) and np.all(codes[~keep] == 0)
+    assert abs(keep.mean() - 0.7) < 0.01
+    plain = torch.from_numpy(x).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(C.dropout_quantize(x, 0.0, seed), plain)
+    # rows 8..15 taken alone draw the words of flat offsets 0.. again: the mask of rows 0..7, not of rows 8..15
+    alone = C.tl_rand(seed, np.arange(8 * 768).reshape(8, 768)) > np.float32(p)
+    assert np.array_equal(alone, keep[:8]) and not np.array_equal(alone, keep[8:16])
+
+
 @pytest.mark.parametrize("k,value", [(20, 1.03125), (20, -0.3), (20, 3.3e-3), (16, 1.00390625 * 1.3), (16, -7.77)])
 def test_sr_recipe_probability_equals_dropped_fraction_exhaustively(k, value):
     t = np.full(1 << k, value, dtype=np.float32)
