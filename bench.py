@@ -61,23 +61,23 @@ def cpu_baseline(cfg, budget_s=12.0):
     }
 
 
-def device_settle(dev, want_ms):
-    """Device conditioning before the warm-up steps: about want_ms milliseconds of the fused step kernel on a separate,
-    small classifier (2 chunks of 16,384 labels, its own weights, inputs and workspace - none of the benchmark's
-    buffers).  When the step kernel starts on a device that was running something else, the first ~25 ms pass through a
-    clock/power transient: over the first 40 launches of a process the same launch takes 0.47, then up to 0.59, then
-    0.45 ms.  A training run is in the settled state; a 20-step measurement right after start-up is not.
-    Returns what was done, for the benchmark's output."""
+def device_settle(dev, want_ms, nc, rows, num_labels, batch, pos_mean, zipf_s):
+    """Device conditioning before the warm-up steps: about want_ms milliseconds of the fused step on a SEPARATE classifier
+    of the benchmark's shape (its own weights, inputs and workspace - none of the benchmark's buffers; freed before the
+    peak-memory counter is reset).  When the step kernel starts on a device that was doing something else, the first
+    ~25 ms pass through a clock/power transient: over the first 40 launches of a process the same launch takes 0.47,
+    then up to 0.59, then 0.45 ms, and only work with the same memory traffic gets the device past it (the same kernel
+    on a classifier that stays in the caches leaves a smaller hump).  A training run is in the settled state; a 20-step
+    measurement right after start-up is not.  Returns what was done, for the benchmark's output."""
     import numpy as np
     import torch
     from elmo_amd import ops, synth
     if want_ms <= 0:
         return {"ms": 0.0, "launches": 0}
-    rows, nc, batch = 16384, 2, 128
     gen = torch.Generator(device=dev).manual_seed(99)
     chunks = [(torch.randn(rows, 768, generator=gen, device=dev) * 0.02).to(torch.float8_e4m3fn) for _ in range(nc)]
     x = torch.from_numpy(synth.make_x(batch, 768, 99)).to(dev).to(torch.bfloat16)
-    labels = torch.from_numpy(synth.make_labels(batch, nc * rows, 5.0, 1.0, 99)).to(dev)
+    labels = torch.from_numpy(synth.make_labels(batch, num_labels, pos_mean, zipf_s, 99)).to(dev)
     ws = ops.alloc_workspace(nc, rows, dev)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -90,7 +90,8 @@ def device_settle(dev, want_ms):
     spent = (time.perf_counter() - t0) * 1e3
     del chunks, x, labels, ws
     torch.cuda.empty_cache()
-    return {"ms": spent, "launches": n, "what": "fused step kernel on a separate 32,768-label classifier (not the benchmark's buffers)"}
+    return {"ms": spent, "launches": n,
+            "what": f"fused step on a separate classifier of the same shape ({nc} x {rows} labels, batch {batch}; not the benchmark's buffers)"}
 
 
 def bench_tiled(args, cfg):
@@ -261,8 +262,8 @@ def main():
     ap.add_argument("--mode", default="step", choices=["step", "forward", "forward_topk"])
     ap.add_argument("--topk-path", default="two_pass", choices=["two_pass", "chunkwise"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--settle-ms", type=float, default=60.0,
-                    help="milliseconds of device conditioning before the warm-up steps (the step kernel on a separate small classifier); 0 = none")
+    ap.add_argument("--settle-ms", type=float, default=100.0,
+                    help="milliseconds of device conditioning before the warm-up steps (the fused step on a separate classifier of the same shape); 0 = none")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only launch the library's plain copy kernel over MIB MiB five times (counter calibration) and exit")
     args = ap.parse_args()
@@ -318,6 +319,7 @@ def main():
     labels = torch.from_numpy(synth.make_labels(cfg.batch, cfg.num_labels, cfg.pos_mean, cfg.zipf_s, cfg.seed)).to(dev)
     torch.cuda.synchronize()
     weight_bytes = sum(c.numel() for c in chunks)
+    settle = device_settle(dev, args.settle_ms, nc, rows, cfg.num_labels, cfg.batch, cfg.pos_mean, cfg.zipf_s)
     torch.cuda.empty_cache()
     torch.cuda.reset_peak_memory_stats()
     base_alloc = torch.cuda.memory_allocated()
@@ -340,7 +342,6 @@ def main():
         assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
         events.append((a, b))
 
-    settle = device_settle(dev, args.settle_ms)
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
