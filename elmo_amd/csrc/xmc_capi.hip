@@ -552,16 +552,16 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       const unsigned short* gsrc = gbl + h0 * g_half;
       floatx4* pdst = partial + h0 * part_half;
       if (weight_type == W_BF16) {
-        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * splits, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_BF16, 2><<<4 * splits, 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_BF16, 2><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
       } else {
-        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * splits, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_E4M3, 2><<<4 * splits, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_E4M3, 2><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
       }
     }
     const int nsub_u = tup_threads(halves) / 256;    // tiles a workgroup of the update kernel works on at a time
-    const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) +
-                      (12 / tup_csteps(halves)) * ((tiles + TUP_TILES * nsub_u - 1) / (TUP_TILES * nsub_u));
+    const int ugroups = (tiles + TUP_TILES * nsub_u - 1) / (TUP_TILES * nsub_u);   // rounded up to eight: see the kernel's index map
+    const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) + (12 / tup_csteps(halves)) * ((ugroups + 7) / 8 * 8);
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
   tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV), stream>>>(                           \
       w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0, partial, part_half, splits,           \

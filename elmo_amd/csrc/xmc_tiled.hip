@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
   if (threadIdx.x == 0) *loss_out = (float)sh[0];
 }
 
-// ---- grad_X partial of one label range: C[128 x 192] = G^T[128 x R] W[R x 192].  blockIdx = fb + 4*split; wavefront w
+// ---- grad_X partial of one label range: C[128 x 192] = G^T[128 x R] W[R x 192].  blockIdx = 8*(4*(split/8) + fb) + split%8; wavefront w
 //      owns features 192fb + 48w.. (3 blocks of 16) against all 8 batch blocks.  Steps of 32 label rows: the step's
 //      slice of W (32 rows x 192 features of this workgroup, whole 16-byte pieces of contiguous row segments) and its
 //      8 KiB of G^T in operand order go straight to LDS, two steps ahead, in a ring of three stages; a compute unit's
@@ -331,7 +331,10 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
   const unsigned lds0 = (unsigned)(size_t)lds;
   const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fb = blockIdx.x & 3, split = blockIdx.x >> 2;
+  // The four workgroups of a label range read the same G^T: they sit on one XCD (workgroups go to the XCDs round robin),
+  // eight apart in launch order, so that three of the four reads are served by that XCD's L2.
+  const int fb = ((int)blockIdx.x >> 3) & 3, split = ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7);
+  if (split * range >= bound) return;   // the grid is rounded up to eight ranges
   floatx4 acc[HV][8][3];
 #pragma unroll
   for (int hv = 0; hv < HV; hv++)
@@ -574,7 +577,10 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tup_lds;
   const int tid = threadIdx.x, wv = (tid >> 6) & 3, sub = tid >> 8, nsub = (int)blockDim.x >> 8;
   const int lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fb = ((int)blockIdx.x - RED_BLOCKS) % NFB, group = ((int)blockIdx.x - RED_BLOCKS) / NFB;   // fb: CS steps of 64 features
+  // fb: CS steps of 64 features.  The NFB workgroups of a tile group read the same rows of G: they sit on one XCD
+  // (workgroups go to the XCDs round robin), eight apart in launch order, and share that XCD's L2.
+  const int jb = (int)blockIdx.x - RED_BLOCKS, fb = (jb >> 3) % NFB, group = ((jb >> 3) / NFB) * 8 + (jb & 7);
+  if (group * TUP_TILES * nsub >= ntiles) return;   // the grid is rounded up to eight tile groups
   // The X^T operand of these features goes to LDS once (it is contiguous in the image) and serves all tiles and
   // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
 #pragma unroll
