@@ -258,7 +258,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="cfg2_fp8_670k")
-    ap.add_argument("--round", default="sr_fast", choices=["sr_fast", "sr_philox", "rtn"])
+    ap.add_argument("--round", default=None, choices=["sr_fast", "sr_philox", "rtn"],
+                    help="default: what the workload names - round to nearest for cfg1_bf16_131k, stochastic for the others "
+                         "(sr_fast where FP8 arithmetic is used, the reference's Philox recipe for bf16 weights and simulated FP8)")
     ap.add_argument("--mode", default="step", choices=["step", "forward", "forward_topk"])
     ap.add_argument("--topk-path", default="two_pass", choices=["two_pass", "chunkwise"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -279,6 +281,8 @@ def main():
     from elmo_amd import _lib, ops, synth
 
     cfg = synth.CONFIGS[args.config]
+    if args.round is None:   # the first workload is defined with round-to-nearest, the others with stochastic rounding
+        args.round = "rtn" if args.config == "cfg1_bf16_131k" else "sr_fast"
     if cfg.batch > ops.MAX_BATCH_TILED:
         print(f"bench.py: config {cfg.name} is not runnable by this build (batch > {ops.MAX_BATCH_TILED})", file=sys.stderr)
         sys.exit(2)

@@ -455,8 +455,9 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
   const size_t halves = (size_t)tiled_halves(max_batch), pairs = (halves + 1) / 2;
+  const size_t rows_buf = (size_t)tiled_group(num_chunks, rows_per_chunk) * rows_pad;   // rows of one launch
   // per batch half G in both orientations; tile_ptr per pair of halves (padded to 64 entries); two loss shares per tile
-  return tiled_layout((int)halves).g + halves * 2 * rows_pad * BP * 2 + pairs * ((tiles + 1 + 63) / 64 * 64 * 4) + (tiles * 8 + 255) / 256 * 256;
+  return tiled_layout((int)halves).g + halves * 2 * rows_buf * BP * 2 + pairs * ((tiles + 1 + 63) / 64 * 64 * 4) + (tiles * 8 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
@@ -491,15 +492,23 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   const int tiles_per_chunk = rows_pad / TL;
   const int num_tiles = num_chunks * tiles_per_chunk;
   const int halves = tiled_halves(batch), pairs = (halves + 1) / 2;   // halves beyond the batch are zero rows of X
+  // Several chunks per launch where they lie one behind the other in memory (the bf16 layer's views of one tensor) and
+  // the compensated head is not in play; the buffers are sized for that many rows either way.
+  const int group_max = tiled_group(num_chunks, rows_per_chunk);
+  int group = kahan_type != 0 ? 1 : group_max;
+  for (int c = 0; c + 1 < num_chunks && group > 1; c++)
+    if ((const unsigned char*)chunk_ptrs[c + 1] != (const unsigned char*)chunk_ptrs[c] + (size_t)rows_per_chunk * D * (weight_type == W_BF16 ? 2 : 1))
+      group = 1;
+  const size_t rows_buf = (size_t)group_max * rows_pad;               // rows the G buffers hold
   const TiledLayout lay = tiled_layout(halves);
   unsigned short* xb = (unsigned short*)(ws + lay.xb);
   unsigned short* xT = (unsigned short*)(ws + lay.xt);
   unsigned* keys = (unsigned*)(ws + lay.keys);
   float* gx_total = (float*)(ws + lay.gx);
   floatx4* partial = (floatx4*)(ws + lay.part);
-  const size_t g_half = 2 * (size_t)rows_pad * BP;    // elements of one half's G and G^T
+  const size_t g_half = 2 * rows_buf * BP;    // elements of one half's G and G^T
   unsigned short* glb = (unsigned short*)(ws + lay.g);
-  unsigned short* gbl = glb + (size_t)rows_pad * BP;
+  unsigned short* gbl = glb + rows_buf * BP;
   int* tile_ptr = (int*)(glb + halves * g_half);
   const size_t tp_stride = (size_t)(num_tiles + 1 + 63) / 64 * 64;   // entries of one pair's tile_ptr
   float* loss_part = (float*)(tile_ptr + pairs * tp_stride);         // one share per sub-tile of 32 rows
@@ -516,17 +525,24 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   }
   tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT,
                                                                         gx_total, loss_part, loss_out ? 2 * num_tiles : 0);
-  for (int c = 0; c < num_chunks; c++) {
+  for (int c = 0; c < num_chunks; c += group) {
     void* w = chunk_ptrs[c];
-    const int rows = c == num_chunks - 1 ? rows_last_chunk : rows_per_chunk;
-    const int rp = (rows + TL - 1) / TL * TL;           // padded rows of this chunk (G buffers use the stride rows_pad)
+    const int nch = c + group <= num_chunks ? group : num_chunks - c;                       // chunks of this launch
+    const int rows = (nch - 1) * rows_per_chunk + (c + nch == num_chunks ? rows_last_chunk : rows_per_chunk);
+    const int rp = (rows + TL - 1) / TL * TL;           // padded rows of this launch (the G buffers use the stride rows_buf)
     const int tiles = rp / TL;
     const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;
-    const unsigned seed = seeds ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c]) : seeds[c]) : 0u;
+    TiledSeeds sd;
+    for (int k = 0; k < T_GROUP; k++)
+      sd.s[k] = seeds && k < nch ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c + k]) : seeds[c + k]) : 0u;
     const int nh = c == 0 ? num_head : 0;   // the compensated head lives in chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127)
-    int range = (rp + T_SPLITS - 1) / T_SPLITS;
+    // label ranges of the grad_X kernel: T_SPLITS slots shared by the launch's chunks, none across a chunk boundary
+    const int cs = nch > 1 ? rows_per_chunk : rp;       // rows of a chunk as the kernels see them
+    const int spc_max = T_SPLITS / nch;
+    int range = (cs + spc_max - 1) / spc_max;
     range = (range + TL - 1) / TL * TL;
-    const int splits = (rp + range - 1) / range;
+    const int spc = (cs + range - 1) / range;            // slots (and at most ranges) per chunk
+    const int splits = nch * spc;
     float* lp = loss_part + 2 * c * tiles_per_chunk;
     for (int hh = 0; hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
@@ -546,17 +562,18 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
         else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
       }
     }
-    // grad_X of the chunk: one pass over W per pair of batch halves, then the fixed-order sums per half
+    // grad_X of the launch's chunks: one pass over W per pair of batch halves, then the fixed-order sums per half
     const size_t part_half = (size_t)T_SPLITS * 4 * 24 * 256;   // floatx4 elements of one half's partials
+    const int ggrid = 4 * ((splits + 7) / 8 * 8);
     for (int h0 = 0; h0 < halves; h0 += 2) {
       const unsigned short* gsrc = gbl + h0 * g_half;
       floatx4* pdst = partial + h0 * part_half;
       if (weight_type == W_BF16) {
-        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_BF16, 2><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<ggrid, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_BF16, 2><<<ggrid, 256, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       } else {
-        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_E4M3, 2><<<4 * ((splits + 7) / 8 * 8), 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, rows_pad, rp, range, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<ggrid, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_E4M3, 2><<<ggrid, 256, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       }
     }
     const int nsub_u = tup_threads(halves) / 256;    // tiles a workgroup of the update kernel works on at a time
@@ -564,7 +581,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) + (12 / tup_csteps(halves)) * ((ugroups + 7) / 8 * 8);
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
   tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV), stream>>>(                           \
-      w, rows, tiles, glb, g_half, xT, lr, seed, saturate, kahan, kahan_type, nh, label0, partial, part_half, splits,           \
+      w, rows, tiles, glb, g_half, xT, lr, sd, cs, saturate, kahan, kahan_type, nh, label0, partial, part_half, nch, spc, range, rp,  \
       weight_type == W_BF16 ? 1 : 0, gx_total)
 #define XMC_LAUNCH_UPDATE_H(WTYPE, RMODE, KH)                                                                                  \
   do {                                                                                                                         \

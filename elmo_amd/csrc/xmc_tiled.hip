@@ -14,6 +14,18 @@ namespace xmc {
 
 enum WType { W_E4M3 = 0, W_BF16 = 1 };
 constexpr int T_SPLITS = 64;                       // label ranges of the grad_X kernel
+constexpr int T_GROUP = 8;                         // most chunks one launch covers
+constexpr int T_GROUP_ROWS = 65536;                // ... and most rows (the G buffers hold the rows of one launch)
+struct TiledSeeds { unsigned s[T_GROUP]; };        // rounding seed of every chunk of a launch
+// Chunks that lie one behind the other in memory and are a multiple of the tile height long are taken several per launch
+// (small chunks leave a launch one tile per compute unit: prologue and tail then dominate).
+__host__ __device__ inline int tiled_group(int num_chunks, int rows_per_chunk) {
+  if (rows_per_chunk % TL != 0) return 1;
+  int g = T_GROUP_ROWS / rows_per_chunk;
+  g = g < T_GROUP ? g : T_GROUP;
+  g = g < num_chunks ? g : num_chunks;
+  return g < 1 ? 1 : g;
+}
 constexpr int T_WS2 = 48 * 2 + 16;                 // LDS row stride of a wavefront's W block, bytes
 
 typedef short tshortx4 __attribute__((ext_vector_type(4)));
@@ -323,9 +335,12 @@ template <int WT, int HV> struct TgxGeom {
   static constexpr int LDS = 3 * STAGE;
 };
 
+//      A launch may cover several chunks that lie one behind the other in memory (cs rows each, a multiple of the tile
+//      height; the last may be shorter): chunk k owns the partial slots k*spc .. k*spc+spc-1, and no label range crosses
+//      a chunk boundary, so that each chunk's sum can be rounded by itself.
 template <int WT, int HV>
-__global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, const unsigned short* gbl,
-                                                          size_t g_half, floatx4* partial, size_t part_half) {
+__global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
+                                                          const unsigned short* gbl, size_t g_half, floatx4* partial, size_t part_half) {
   typedef TgxGeom<WT, HV> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
@@ -334,7 +349,9 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
   // The four workgroups of a label range read the same G^T: they sit on one XCD (workgroups go to the XCDs round robin),
   // eight apart in launch order, so that three of the four reads are served by that XCD's L2.
   const int fb = ((int)blockIdx.x >> 3) & 3, split = ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7);
-  if (split * range >= bound) return;   // the grid is rounded up to eight ranges
+  const int ck = split / spc, lbeg = ck * cs + (split - ck * spc) * range;
+  const int cend = min((ck + 1) * cs, bound);   // bound: the launch's rows rounded up to a tile
+  if (lbeg >= cend) return;                     // the grid is rounded up to eight ranges; a short last chunk has fewer
   floatx4 acc[HV][8][3];
 #pragma unroll
   for (int hv = 0; hv < HV; hv++)
@@ -342,8 +359,8 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
     for (int mb = 0; mb < 8; mb++)
 #pragma unroll
       for (int nn = 0; nn < 3; nn++) acc[hv][mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const int lbeg = split * range, lend = min(lbeg + range, bound);   // bound: this chunk's rows rounded up to a tile
-  const int nsteps = lend > lbeg ? (lend - lbeg + 31) >> 5 : 0;
+  const int lend = min(lbeg + range, cend);
+  const int nsteps = (lend - lbeg + 31) >> 5;
   // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv+4, ...; indices past the last piece repeat it),
   // so that "all but the newest PER_WAVE" means the step before has landed.  Steps past the end repeat the last one.
   auto issue_step = [&](int st, int stage) {
@@ -426,27 +443,34 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
 // in the first workgroups of the chunk's update launch (the two do not depend on each other), so the sum costs no
 // launch of its own and hides behind the update.
 constexpr int TRED_WAVES = 384;
-__device__ __forceinline__ void tiled_reduce_wave(int widx, int lane, const floatx4* partial, int splits, int round_bf16, float* gx_total) {
+__device__ __forceinline__ void tiled_reduce_wave(int widx, int lane, const floatx4* partial, int nchunks, int spc, int cs, int range,
+                                                  int bound, int round_bf16, float* gx_total) {
   // (slot, fb, wavefront of the grad_X kernel's layout); eight loads in flight
   const int slot = widx >> 4, fb = (widx >> 2) & 3, wv = widx & 3;
   const int tid = wv * 64 + lane, l16 = lane & 15, kg = lane >> 4;
-  floatx4 s = {0.f, 0.f, 0.f, 0.f};
-  int sp = 0;
-  for (; sp + 8 <= splits; sp += 8) {
-    floatx4 v[8];
-#pragma unroll
-    for (int x = 0; x < 8; x++) v[x] = partial[(((size_t)(sp + x) * 4 + fb) * 24 + slot) * 256 + tid];
-#pragma unroll
-    for (int x = 0; x < 8; x++) s += v[x];
-  }
-  for (; sp < splits; sp++) s += partial[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
   const int mb = slot / 3, nn = slot - mb * 3;
   const int col = 192 * fb + 48 * wv + 16 * nn + l16;
+  floatx4 tot = {0.f, 0.f, 0.f, 0.f};
+  for (int ck = 0; ck < nchunks; ck++) {   // the chunks of the launch, each summed (and rounded) by itself
+    const int crows = min((ck + 1) * cs, bound) - ck * cs, splits = (crows + range - 1) / range;
+    const floatx4* pc = partial + (size_t)ck * spc * 4 * 24 * 256;
+    floatx4 s = {0.f, 0.f, 0.f, 0.f};
+    int sp = 0;
+    for (; sp + 8 <= splits; sp += 8) {
+      floatx4 v[8];
+#pragma unroll
+      for (int x = 0; x < 8; x++) v[x] = pc[(((size_t)(sp + x) * 4 + fb) * 24 + slot) * 256 + tid];
+#pragma unroll
+      for (int x = 0; x < 8; x++) s += v[x];
+    }
+    for (; sp < splits; sp++) s += pc[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
+#pragma unroll
+    for (int i = 0; i < 4; i++) tot[i] += round_bf16 ? bf16_rt(s[i]) : s[i];
+  }
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int b = 16 * mb + 4 * kg + i;
-    const float v = round_bf16 ? bf16_rt(s[i]) : s[i];
-    gx_total[(size_t)b * D + col] += v;
+    gx_total[(size_t)b * D + col] += tot[i];
   }
 }
 
@@ -560,17 +584,17 @@ constexpr int tup_lds_bytes(int halves) { return halves * tup_xbytes(halves); }
 // branches around the products the compiler issued every LDS operand read right in front of its matrix instruction.
 template <int WT, int MODE, int HALVES, bool KAHAN>
 __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES == 2 ? 2 : 1) void tiled_update_kernel(
-    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, unsigned seed,
-    int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
-    int red_splits, int red_round_bf16, float* red_total) {
+    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, TiledSeeds seeds,
+    int cs, int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
+    int red_nchunks, int red_spc, int red_range, int red_bound, int red_round_bf16, float* red_total) {
   static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
   // the first workgroups sum the chunk's grad_X partials (384 wavefronts per batch half), the others update the weights
   constexpr int CS = tup_csteps(HALVES), XB = tup_xbytes(HALVES), NFB = 12 / CS, WAVES = tup_threads(HALVES) / 64;
   constexpr int RED_BLOCKS = TRED_WAVES * HALVES / WAVES;
   if ((int)blockIdx.x < RED_BLOCKS) {
     const int widx = (int)blockIdx.x * WAVES + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
-    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_splits, red_round_bf16,
-                      red_total + (size_t)hh * BP * D);
+    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
+                      red_range, red_bound, red_round_bf16, red_total + (size_t)hh * BP * D);
     return;
   }
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
@@ -618,7 +642,12 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
   const int row = tile * TL + 16 * wv + l16;
   const bool live = row < rows;
   const bool head = KAHAN && kahan_type != 0 && row < num_head;
-  const int orow = (WT == W_E4M3 && !head) ? row - num_head : row;   // row of the random offset
+  // the launch may cover several chunks of cs rows (a multiple of the tile height): the tile's chunk gives the seed, and
+  // the random offsets count rows from the chunk's first
+  const int ck = __builtin_amdgcn_readfirstlane((tile * TL) / cs);
+  const unsigned seed = seeds.s[ck];
+  const int crow = row - ck * cs;
+  const int orow = (WT == W_E4M3 && !head) ? crow - num_head : crow;   // row of the random offset
   bf16x8 gf[HALVES][4];
   intx4 wr_t[CS][WDW / 4];
 #pragma unroll

@@ -505,3 +505,49 @@ def test_true_fp8_arithmetic_at_batch_512(gpu):
         d = H.e4m3_ulp_distance(a, b)
         assert d.max() <= 1 and (d != 0).mean() < 5e-3
     check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx)
+
+
+@pytest.mark.parametrize("L,nc,batch,mode", [
+    (4096, 4, 32, "rtn"),             # four chunks of 1,024 rows in one launch
+    (4093, 4, 48, "rtn"),             # the last chunk three rows short
+    (10240, 10, 16, "sr_philox"),     # ten chunks: launches of eight and two; a seed per chunk
+    (2048, 2, 200, "sr_philox"),      # two batch halves
+    (64 * 1200, 2, 16, "rtn"),        # chunks above the row budget of a launch stay one per launch
+])
+def test_bf16_layer_with_several_chunks_per_launch(gpu, L, nc, batch, mode):
+    """Chunks that are a multiple of 64 rows long and lie one behind the other in memory (the bf16 layer's views) are taken
+    several per launch: same results as the oracle's chunk-by-chunk step - per-chunk seeds and random offsets, the
+    per-chunk bf16 rounding of grad_X."""
+    x, w, labels = bf16_case(L, batch, 300 + nc)
+    seeds = [1000 + 7 * c for c in range(nc)] if mode != "rtn" else None
+    new, gf, gb = run_bf16(x, w, labels, nc, gpu, mode, seeds)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.05, nc, seeds=seeds, sr_mode="rtn" if mode == "rtn" else "reference")
+    check_bf16_weights(new, ref_w, w, x)
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+    if mode != "rtn":
+        # a seed that belongs to another chunk would show: the same step with the seeds rotated differs in every chunk
+        new2, _, _ = run_bf16(x, w, labels, nc, gpu, mode, seeds[1:] + seeds[:1])
+        cs = (L + nc - 1) // nc
+        for c in range(nc):
+            assert (new2[c * cs:(c + 1) * cs] != new[c * cs:(c + 1) * cs]).mean() > 0.1
+
+
+@pytest.mark.parametrize("mode,quant", [("sr_philox", False), ("sr_fast", True), ("rtn", False)])
+def test_e4m3_chunks_in_one_allocation_take_one_launch(gpu, mode, quant):
+    """e4m3 chunks that are views of one tensor (1,024 rows each) against the same chunks as separate tensors, which run one
+    per launch: bit-equal weights and grad_X bits (the partial sums keep their order within a chunk; across chunks the
+    fp32 totals are added in the same order)."""
+    import torch
+    from elmo_amd import ops
+    nc, rows, batch = 3, 1024, 256 if quant else 64
+    case = H.make_case(nc, rows, batch, 77)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    whole = torch.cat(chunks).contiguous()
+    views = [whole[c * rows:(c + 1) * rows] for c in range(nc)]
+    seeds = [5, 6, 7]
+    kw = dict(seeds=None if mode == "rtn" else seeds, round_mode=mode, want_f32=True, quantize_x=quant, saturate=quant)
+    g1, gf1 = ops.tiled_step(views, rows, "e4m3", x, labels, 0.05, **kw)
+    g0, gf0 = ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.05, **kw)
+    assert torch.equal(torch.cat(chunks).view(torch.uint8), whole.view(torch.uint8))
+    assert torch.equal(g0.view(torch.int16), g1.view(torch.int16))
+    assert torch.allclose(gf0, gf1, rtol=0, atol=1e-6 * float(gf0.abs().max()))
