@@ -51,6 +51,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
 #define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
     XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false);
@@ -523,8 +524,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys + (size_t)pr * MAX_POS, n_pad, rows_per_chunk, tiles_per_chunk,
                                                                   num_tiles, tile_ptr + pr * tp_stride);
   }
-  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x, xb, xT,
-                                                                        gx_total, loss_part, loss_out ? 2 * num_tiles : 0);
+  // true-FP8 arithmetic with two or four batch halves: FP8 matrix products, the logits of a pair of halves in one pass
+  const bool fp8_logits = weight_type == W_E4M3 && quantize_x && halves >= 2 && !loss_out;
+  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x,
+                                                                        fp8_logits ? 1 : 0, xb, xT, gx_total, loss_part,
+                                                                        loss_out ? 2 * num_tiles : 0);
   for (int c = 0; c < num_chunks; c += group) {
     void* w = chunk_ptrs[c];
     const int nch = c + group <= num_chunks ? group : num_chunks - c;                       // chunks of this launch
@@ -544,7 +548,13 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int spc = (cs + range - 1) / range;            // slots (and at most ranges) per chunk
     const int splits = nch * spc;
     float* lp = loss_part + 2 * c * tiles_per_chunk;
-    for (int hh = 0; hh < halves; hh++) {
+    for (int hh = 0; fp8_logits && hh < halves; hh += 2) {
+      const int nsub = 2 * tiles, lgrid = nsub < di.cus ? nsub : di.cus;
+      tiled_logits_fp8_kernel<<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(
+          w, rows, nsub, (const unsigned char*)xb + (size_t)hh * BP * D, keys + (size_t)(hh >> 1) * MAX_POS,
+          tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk, label0, glb + hh * g_half, gbl + hh * g_half, g_half);
+    }
+    for (int hh = 0; !fp8_logits && hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
       unsigned short* gb = gbl + hh * g_half;
       const unsigned short* xh = xb + (size_t)hh * BP * D;

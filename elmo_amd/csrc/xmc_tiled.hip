@@ -77,8 +77,10 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 //   xT: X^T for grad_W (never quantised): block (fblk, ks) = 16 features x batch rows 32ks.., the features of a block
 //       chosen so that a lane of the update kernel owns consecutive ones
 // (also clears the fp32 grad_X total, one entry per thread, and the loss shares if there are any: no launches for that)
-__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, unsigned short* xb, unsigned short* xT,
-                                    float* gx_total, float* loss_part, int n_loss) {
+// fp8_image: instead of the bf16 image, xb receives the e4m3 codes in the B-operand order of v_mfma_f32_16x16x128_f8f6f4
+// (per half: [(16-row block)*6 + ks][lane = row % 16 + 16*((k / 32) % 4)][32 bytes], k = 128 ks + 32 (lane / 16) + byte).
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, int fp8_image, unsigned short* xb,
+                                    unsigned short* xT, float* gx_total, float* loss_part, int n_loss) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
   gx_total[i] = 0.f;
@@ -86,14 +88,19 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
   int b = i / D, k = i - b * D;
   unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
   unsigned short vq = v;
+  int code = 0;
   if (quantize) {
     const float f = clamp448(bf16_from_bits(v));
-    const int code = __builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false);
+    code = __builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false);
     const floatx2 back = __builtin_amdgcn_cvt_pk_f32_fp8(code, false);
     vq = bf16_bits(back.x);
   }
   const int half = b >> 7, bh = b & 127;
-  xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
+  if (fp8_image)
+    ((unsigned char*)xb)[(size_t)half * BP * D + ((size_t)((bh >> 4) * 6 + (k >> 7)) * 64 + (bh & 15) + 16 * ((k >> 5) & 3)) * 32 + (k & 31)] =
+        (unsigned char)(code & 0xFF);
+  else
+    xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
   // feature k = 192 fbk + 64 c + 16 kgk + 4 q + e sits in row 4 kgk + e of block 12 fbk + 4 c + q: in the update kernel
   // a lane then owns 16 consecutive features per step c, and the four lanes of a label row 64 consecutive bytes
   const int fbk = k / 192, r = k - fbk * 192, kgk = (r >> 4) & 3, nn = 4 * (r >> 6) + ((r >> 2) & 3), e = r & 3;
@@ -296,6 +303,144 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
       if (lane == 0) wsum[v] = lsum;
       __syncthreads();
       if (tid == 0) loss_part[st] += ((wsum[0] + wsum[1]) + (wsum[2] + wsum[3])) + ((wsum[4] + wsum[5]) + (wsum[6] + wsum[7]));
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last loads still target LDS
+}
+
+// ---- the same for the true-FP8 arithmetic with two batch halves per pass: the logits of e4m3 weights against e4m3(X)
+//      are FP8 matrix products (chunked_fp8xmc_clf.py:101-102), so the rows go from LDS into v_mfma_f32_16x16x128_f8f6f4
+//      as they are (no widening to bf16, a quarter of the matrix instructions per batch row) and wavefront v keeps the
+//      e4m3 operand of batch rows 16v.. of BOTH halves (96 registers, as the bf16 operand of one half took): one pass over
+//      the weights yields the G of 256 batch rows.  Tile loop, positives, rounding and both layouts of G as above; the
+//      products are exact in fp32 either way, only the order of the fp32 sums differs from the bf16 form.
+//      xq: e4m3 image of the pair's X in B-operand order, [half][(16-row block)*6 + ks][lane][32 bytes] (tiled_prep_x_kernel)
+__global__ __launch_bounds__(512, 1) void tiled_logits_fp8_kernel(const void* w, int rows, int nsub, const unsigned char* xq,
+                                                                  const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
+                                                                  unsigned short* glb, unsigned short* gbl, size_t g_half) {
+  typedef TlgGeom<W_E4M3> G;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tlg_lds[];
+  __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tlg_lds;
+  const int tid = threadIdx.x, v = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const __attribute__((address_space(4))) unsigned* ckeys = (const __attribute__((address_space(4))) unsigned*)keys;
+  const __attribute__((address_space(4))) int* ctile_ptr = (const __attribute__((address_space(4))) int*)tile_ptr;
+  int prow[G::PER_WAVE], pcol[G::PER_WAVE];
+#pragma unroll
+  for (int s = 0; s < G::PER_WAVE; s++) {
+    const int slot = (v + 8 * s) * 64 + lane;
+    prow[s] = min(slot / G::SLOTS, TLG_ROWS - 1);
+    pcol[s] = min(slot - (slot / G::SLOTS) * G::SLOTS, G::SLOTS - 2) * 16;
+  }
+  auto issue_sub = [&](int st, int buf) {
+    const int s0 = min(st, nsub - 1) * TLG_ROWS;
+#pragma unroll
+    for (int s = 0; s < G::PER_WAVE; s++) {
+      if (v + 8 * s < G::PIECES) {
+        const int lr = min(s0 + prow[s], rows - 1);
+        t_lds_load16((const unsigned char*)w + (size_t)lr * G::ROWB + pcol[s], (unsigned)(buf * G::BUF + (v + 8 * s) * 1024));
+      }
+    }
+  };
+  const float nlog2e = -1.44269504088896340736f;
+  const int gs = (int)gridDim.x;
+  __attribute__((address_space(3))) unsigned char* stg = lds + G::STAGE0 + v * 1024;
+  issue_sub(blockIdx.x, 0);
+  issue_sub(blockIdx.x + gs, 1);
+  intx8 xr[2][6];   // the e4m3 operands of this wavefront's batch rows in either half
+#pragma unroll
+  for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++) xr[hf][ks] = *(const intx8*)(xq + (size_t)hf * BP * D + ((size_t)(v * 6 + ks) * 64 + lane) * 32);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // from here on the loop counts its own operations: nothing is in flight
+  int it = 0, b0 = 0, b2 = 2;   // it % 3, (it + 2) % 3
+  for (int st = blockIdx.x; st < nsub; st += gs, it++) {
+    // younger than the loads of this sub-tile: the loads of the next one and the stores of up to two steps (six per
+    // wavefront and step: per half two of G^T and one of G)
+    if (it == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN) : "memory");
+    else if (it == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 6) : "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 12) : "memory");
+    const int p0 = ctile_ptr[st >> 1], p1 = ctile_ptr[(st >> 1) + 1];
+    __syncthreads();
+    issue_sub(st + 2 * gs, b2);
+    const int buf = b0;
+    b0 = b0 == 2 ? 0 : b0 + 1;
+    b2 = b2 == 2 ? 0 : b2 + 1;
+    floatx4 acc[2][2];   // [label block][half]
+#pragma unroll
+    for (int lb = 0; lb < 2; lb++) { acc[lb][0] = floatx4{0.f, 0.f, 0.f, 0.f}; acc[lb][1] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+    const unsigned abase = (unsigned)(buf * G::BUF + l16 * G::STRIDE + kg * 32);
+    auto rd = [&](int ks, int lb) {
+      const __attribute__((address_space(3))) intx4* q = (const __attribute__((address_space(3))) intx4*)(lds + abase + lb * 16 * G::STRIDE + ks * 128);
+      const intx4 lo = q[0], hi = q[1];
+      return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    intx8 araw[3][2];   // the LDS reads run two K steps ahead of the matrix instructions
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) { araw[ks][0] = rd(ks, 0); araw[ks][1] = rd(ks, 1); }
+#pragma unroll
+    for (int ks = 0; ks < 6; ks++) {
+      if (ks + 2 < 6) { araw[(ks + 2) % 3][0] = rd(ks + 2, 0); araw[(ks + 2) % 3][1] = rd(ks + 2, 1); }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int lb = 0; lb < 2; lb++)
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+          acc[lb][hf] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(araw[ks % 3][lb], xr[hf][ks], acc[lb][hf], 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // acc[lb][hf][e] = Z[label 32 st + 16 lb + 4kg + e][batch 128 hf + 16v + l16]
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+      float sg[2][4];
+#pragma unroll
+      for (int lb = 0; lb < 2; lb++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          sg[lb][e] = bf16_rt(__builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(bf16_rt(acc[lb][hf][e]) * nlog2e)));
+      // positives of the enclosing 64-row tile, as in tiled_logits_kernel; the keys hold the row within the pair of halves
+      if (p1 > p0) {
+        typedef unsigned t_keysx8 __attribute__((ext_vector_type(8), aligned(4)));
+        const unsigned lbase = label0_chunk + (unsigned)(st * TLG_ROWS);
+        unsigned prev = p0 > 0 ? ckeys[p0 - 1] : ~ckeys[p0];
+        for (int e0 = p0; e0 < p1; e0 += 8) {
+          const t_keysx8 kk = *(const __attribute__((address_space(4))) t_keysx8*)(ckeys + e0);
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            const unsigned key = kk[j];
+            const unsigned lrel = (key >> 8) - lbase;                  // label within the sub-tile
+            const unsigned b = (key & 255u) - (unsigned)(BP * hf);     // batch row within this half
+            if (e0 + j < p1 && key != prev && lrel < (unsigned)TLG_ROWS && (b >> 4) == (unsigned)v) {
+              const bool mine = (unsigned)kg == ((lrel >> 2) & 3u) && (unsigned)l16 == (b & 15u);
+              const unsigned sel = ((lrel >> 4) << 2) | (lrel & 3u);
+#pragma unroll
+              for (int c = 0; c < 8; c++)
+                if (sel == (unsigned)c) sg[c >> 2][c & 3] = mine ? bf16_rt(sg[c >> 2][c & 3] - 1.0f) : sg[c >> 2][c & 3];
+            }
+            prev = key;
+          }
+        }
+      }
+      unsigned short* gl = glb + (size_t)hf * g_half;
+      unsigned short* gb = gbl + (size_t)hf * g_half;
+#pragma unroll
+      for (int lb = 0; lb < 2; lb++) {
+        const int r0 = st * TLG_ROWS + 16 * lb;
+        unsigned short sb[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) sb[e] = (r0 + 4 * kg + e < rows) ? bf16_bits(sg[lb][e]) : (unsigned short)0;
+        uint2 o;
+        o.x = (unsigned)sb[0] | ((unsigned)sb[1] << 16);
+        o.y = (unsigned)sb[2] | ((unsigned)sb[3] << 16);
+        *(uint2*)(gb + ((size_t)(st * 8 + v) * 64 + l16 + 16 * (2 * lb + (kg >> 1))) * 8 + 4 * (kg & 1)) = o;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          *(__attribute__((address_space(3))) unsigned short*)(stg + (16 * lb + 4 * kg + e) * 32 + 2 * l16) = sb[e];
+      }
+      {
+        const int lbo = lane >> 5, half = (lane >> 4) & 1;
+        const intx4 gq = *(const __attribute__((address_space(3))) intx4*)(stg + (lane & 15) * 32 + 512 * lbo + 16 * half);
+        *(intx4*)(gl + ((size_t)((2 * st + lbo) * 4 + (v >> 1)) * 64 + (lane & 15) + 16 * (2 * (v & 1) + half)) * 8) = gq;
+      }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last loads still target LDS
