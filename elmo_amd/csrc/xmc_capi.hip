@@ -52,6 +52,9 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
     (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
+    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
+    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
     // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
 #define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
     XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false);
@@ -526,9 +529,11 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   }
   // true-FP8 arithmetic with two or four batch halves: FP8 matrix products, the logits of a pair of halves in one pass
   const bool fp8_logits = weight_type == W_E4M3 && quantize_x && halves >= 2 && !loss_out;
+  // e4m3 weights, two batch halves, no compensated head: the feature-split update kernel (X^T in registers)
+  const bool split_update = weight_type == W_E4M3 && halves == 2 && kahan_type == 0;
   tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x,
-                                                                        fp8_logits ? 1 : 0, xb, xT, gx_total, loss_part,
-                                                                        loss_out ? 2 * num_tiles : 0);
+                                                                        fp8_logits ? 1 : 0, split_update ? 1 : 0, xb, xT, gx_total,
+                                                                        loss_part, loss_out ? 2 * num_tiles : 0);
   for (int c = 0; c < num_chunks; c += group) {
     void* w = chunk_ptrs[c];
     const int nch = c + group <= num_chunks ? group : num_chunks - c;                       // chunks of this launch
@@ -600,7 +605,18 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     else XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, 4, KH);                                                                             \
   } while (0)
     const bool with_head = kahan_type != 0 && nh > 0;   // only chunk 0 of the head-Kahan layer
-    if (weight_type == W_BF16) {
+    if (split_update) {
+      int streams = (tiles + 7) / 8 * 8;
+      streams = streams < 128 ? streams : 128;           // two workgroups per compute unit, four per stream
+      const int grid2 = TRED_WAVES * 2 / 4 + 4 * streams;
+#define XMC_LAUNCH_UPDATE2(RMODE)                                                                                              \
+  tiled_update2_kernel<RMODE><<<grid2, 256, 2 * TU2_GBUF, stream>>>(w, rows, tiles, glb, g_half, (const bf16x8*)xT, lr, sd, cs, saturate, \
+                                                                    label0, partial, part_half, nch, spc, range, rp, gx_total)
+      if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE2(ROUND_RTN);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE2(ROUND_SR_FAST);
+      else XMC_LAUNCH_UPDATE2(ROUND_SR_PHILOX);
+#undef XMC_LAUNCH_UPDATE2
+    } else if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_RTN, false);
       else XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_SR_PHILOX, false);
     } else if (with_head) {

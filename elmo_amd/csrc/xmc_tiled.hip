@@ -79,8 +79,10 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 // (also clears the fp32 grad_X total, one entry per thread, and the loss shares if there are any: no launches for that)
 // fp8_image: instead of the bf16 image, xb receives the e4m3 codes in the B-operand order of v_mfma_f32_16x16x128_f8f6f4
 // (per half: [(16-row block)*6 + ks][lane = row % 16 + 16*((k / 32) % 4)][32 bytes], k = 128 ks + 32 (lane / 16) + byte).
-__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, int fp8_image, unsigned short* xb,
-                                    unsigned short* xT, float* gx_total, float* loss_part, int n_loss) {
+// xt_split (two halves only): xT in the order of tiled_update2_kernel instead, [feature quarter][wavefront][block cg][K step
+// of 32 batch rows, 8 over both halves][lane][8], row 4kq + e of block cg being feature 12kq + 4cg + e of the wavefront's 48.
+__global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, int fp8_image, int xt_split,
+                                    unsigned short* xb, unsigned short* xT, float* gx_total, float* loss_part, int n_loss) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
   gx_total[i] = 0.f;
@@ -104,7 +106,12 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
   // feature k = 192 fbk + 64 c + 16 kgk + 4 q + e sits in row 4 kgk + e of block 12 fbk + 4 c + q: in the update kernel
   // a lane then owns 16 consecutive features per step c, and the four lanes of a label row 64 consecutive bytes
   const int fbk = k / 192, r = k - fbk * 192, kgk = (r >> 4) & 3, nn = 4 * (r >> 6) + ((r >> 2) & 3), e = r & 3;
-  xT[(size_t)half * BP * D + ((size_t)((fbk * 12 + nn) * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
+  if (xt_split) {
+    const int wq = r / 48, c48 = r - wq * 48, kq = c48 / 12, rem = c48 - kq * 12, cg = rem >> 2, rr = 4 * kq + (rem & 3);
+    xT[((size_t)((((fbk * 4 + wq) * 3 + cg) * 8 + (b >> 5)) * 64 + rr + 16 * ((b >> 3) & 3))) * 8 + (b & 7)] = v;
+  } else {
+    xT[(size_t)half * BP * D + ((size_t)((fbk * 12 + nn) * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
+  }
 }
 
 __global__ void tiled_zero_kernel(float* p, int n) {
@@ -873,6 +880,133 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
     }
   }
   }
+}
+
+
+// ---- grad_W and the update for e4m3 weights and two batch halves, feature-split: in tiled_update_kernel a wavefront
+//      owns 16 label rows and takes the X^T operand of every matrix instruction from LDS (96 reads of 1 KiB per tile, the
+//      same ones in the four wavefronts of a tile: with 256 batch rows the LDS is the limit).  Here a wavefront owns 48
+//      features of the workgroup's quarter and keeps their X^T operand for all 256 batch rows in registers (96 of them);
+//      the tile's G - 32 KiB, already in operand order in memory - goes straight to LDS once per workgroup, two buffers,
+//      and every wavefront reads its 32 blocks from there: a third of the LDS traffic.  A^T[48 features x 16 rows] per
+//      row block, the features of a block permuted (row 4kg + e of block cg is feature 12kg + 4cg + e of the 48, see
+//      tiled_prep_x_kernel) so that a lane ends up with 12 consecutive bytes of one weight row.  Persistent: stream s of
+//      the launch walks tiles s, s + streams, ...; its four workgroups (one per feature quarter) sit on one XCD, eight
+//      apart in launch order, and share the tile's G through that XCD's L2.  The first workgroups sum the grad_X
+//      partials, as in tiled_update_kernel.  Same arithmetic, rounding modes and random words as there.
+constexpr int TU2_GBUF = 32768;   // one tile's G: [half][row block][K step] blocks of 1 KiB
+template <int MODE>
+__global__ __launch_bounds__(256, 2) void tiled_update2_kernel(
+    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half, const bf16x8* xt2, float lr, TiledSeeds seeds, int cs,
+    int saturate, unsigned label0, const floatx4* red_partial, size_t red_part_half, int red_nchunks, int red_spc, int red_range,
+    int red_bound, float* red_total) {
+  constexpr int RED_BLOCKS = TRED_WAVES * 2 / 4;
+  if ((int)blockIdx.x < RED_BLOCKS) {
+    const int widx = (int)blockIdx.x * 4 + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
+    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
+                      red_range, red_bound, 0, red_total + (size_t)hh * BP * D);
+    return;
+  }
+  extern __shared__ __attribute__((aligned(16))) unsigned char tu2_lds[];
+  __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tu2_lds;
+  const unsigned lds0 = (unsigned)(size_t)lds;
+  const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int jb = (int)blockIdx.x - RED_BLOCKS, fb = (jb >> 3) & 3, stream = (jb >> 5) * 8 + (jb & 7);
+  const int nstreams = (((int)gridDim.x - RED_BLOCKS) >> 5) * 8;
+  if (stream >= ntiles) return;
+  bf16x8 xt[3][8];   // X^T of this wavefront's 48 features: feature blocks x K steps of 32 batch rows (both halves)
+#pragma unroll
+  for (int cg = 0; cg < 3; cg++)
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) xt[cg][ks] = xt2[(size_t)((((fb * 4 + wv) * 3 + cg) * 8 + ks) * 64 + lane)];
+  // the tile's G: per half 16 KiB of consecutive memory; wavefront wv fetches pieces wv, wv + 4, ...
+  auto issue_g = [&](int t, int buf) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int p = wv + 4 * j, hf = p >> 4, q = p & 15;
+      t_lds_load16((const unsigned char*)(glb + (size_t)hf * g_half + ((size_t)t * 16 + q) * 512) + lane * 16,
+                   lds0 + (unsigned)(buf * TU2_GBUF + p * 1024));
+    }
+  };
+  const int col0 = 192 * fb + 48 * wv + 12 * kg;   // this lane's 12 features
+  // The weights come in through inline assembly like the pieces of G, so that the compiler counts none of the loads of
+  // this loop and the waits below are the only ones: rows past the end read the last valid row (their result is not
+  // stored).
+  typedef unsigned tu2_x3 __attribute__((ext_vector_type(3)));
+  auto load_w = [&](int t, tu2_x3 (&wr)[4]) {
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+      const int row = min(t * TL + 16 * rb + l16, rows - 1);
+      const unsigned char* src = (const unsigned char*)w + (size_t)row * D + col0;
+      asm volatile("global_load_dwordx3 %0, %1, off" : "=v"(wr[rb]) : "v"(src) : "memory");
+    }
+  };
+  tu2_x3 wn[4];
+  issue_g(stream, 0);
+  load_w(stream, wn);
+  int buf = 0;
+  bool prev_full = false;   // the tile before stored all four row blocks: four stores are younger than this tile's loads
+#pragma unroll 1
+  for (int t = stream; t < ntiles; t += nstreams) {
+    // This wavefront's pieces of G(t) and the weights of tile t have arrived (memory operations complete in order: all
+    // but the four stores of the tile before, when it had that many); behind the barrier every wavefront's pieces are
+    // there and nobody reads the other buffer any more.
+    if (prev_full) asm volatile("s_waitcnt vmcnt(4)" : "+v"(wn[0]), "+v"(wn[1]), "+v"(wn[2]), "+v"(wn[3]) : : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" : "+v"(wn[0]), "+v"(wn[1]), "+v"(wn[2]), "+v"(wn[3]) : : "memory");
+    __syncthreads();
+    prev_full = (t + 1) * TL <= rows;
+    unsigned wc[4][3];
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++)
+#pragma unroll
+      for (int cg = 0; cg < 3; cg++) wc[rb][cg] = wn[rb][cg];
+    if (t + nstreams < ntiles) {
+      issue_g(t + nstreams, buf ^ 1);
+      load_w(t + nstreams, wn);
+    }
+    // the launch may cover several chunks of cs rows (a multiple of the tile height): the tile's chunk gives the seed, and
+    // the random offsets count rows from the chunk's first
+    const int ck = __builtin_amdgcn_readfirstlane((t * TL) / cs);
+    const unsigned seed = seeds.s[ck];
+    const __attribute__((address_space(3))) unsigned char* gt = lds + buf * TU2_GBUF + lane * 16;
+    // the products of row block rb + 1 are issued in front of the update of row block rb: they run in the matrix pipe
+    // while the vector instructions of the update go through
+    auto products = [&](int rb, floatx4 (&a)[3]) {
+      bf16x8 bg[8];
+#pragma unroll
+      for (int k8 = 0; k8 < 8; k8++)
+        bg[k8] = *(const __attribute__((address_space(3))) bf16x8*)(gt + ((k8 >> 2) * 16 + rb * 4 + (k8 & 3)) * 1024);
+#pragma unroll
+      for (int cg = 0; cg < 3; cg++) a[cg] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k8 = 0; k8 < 8; k8++)
+#pragma unroll
+        for (int cg = 0; cg < 3; cg++) a[cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][k8], bg[k8], a[cg], 0, 0, 0);
+    };
+    floatx4 acc[2][3];
+    products(0, acc[0]);
+#pragma unroll
+    for (int rb = 0; rb < 4; rb++) {
+      if (rb + 1 < 4) products(rb + 1, acc[(rb + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      const floatx4 (&a)[3] = acc[rb & 1];
+      // a[cg][e] = A[label row 16rb + l16][feature col0 + 4cg + e]
+      const int row = t * TL + 16 * rb + l16, orow = row - ck * cs;
+      if (row < rows) {
+        unsigned wo[3];
+#pragma unroll
+        for (int cg = 0; cg < 3; cg++)
+          t_update4<W_E4M3, MODE>(a[cg], &wc[rb][cg], nullptr, false, 0, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * cg),
+                                  (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * cg) >> 2), seed, saturate, &wo[cg],
+                                  nullptr);
+        unsigned* dst = (unsigned*)((unsigned char*)w + (size_t)row * D + col0);
+        dst[0] = wo[0]; dst[1] = wo[1]; dst[2] = wo[2];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    buf ^= 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace xmc
