@@ -473,15 +473,17 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
 //      8 KiB of G^T in operand order go straight to LDS, two steps ahead, in a ring of three stages; a compute unit's
 //      memory path handles few cache lines per clock, and register loads in operand order touched four times as many.
 //      The W operand comes back transposed (ds_read_b64_tr_b8 + exact fp8->bf16, or ds_read_b64_tr_b16).
-//      With two batch halves (HV = 2) one pass over W serves both: the step's G^T of either half is staged, the W
-//      operand is read and converted once, and every wavefront keeps the accumulators of both halves.
+//      With two batch halves (HV = 2) one pass over W serves both: the step's G^T of either half is staged, and the
+//      workgroup has eight wavefronts, four per half (two per SIMD: one's LDS reads and conversions run under the
+//      other's matrix instructions; with both halves' accumulators in one wavefront a SIMD had a single wavefront).
 template <int WT, int HV> struct TgxGeom {
   static constexpr int ROWB = WT == W_BF16 ? 384 : 192;                  // bytes of this workgroup's features in one row
   static constexpr int STRIDE = ROWB + 16;                                // LDS row stride
   static constexpr int SLOTS = STRIDE / 16;                               // 16-byte slots per LDS row, the last one padding
   static constexpr int WPIECES = (32 * SLOTS + 63) / 64;                  // wave-wide loads of the W slice (7 or 13)
   static constexpr int PIECES = WPIECES + 8 * HV;                         // ... and of G^T (8 per batch half)
-  static constexpr int PER_WAVE = (PIECES + 3) / 4;                       // every wavefront issues this many per step (4 or 6)
+  static constexpr int WAVES = 4 * HV;                                    // four wavefronts (48 features each) per batch half
+  static constexpr int PER_WAVE = (PIECES + WAVES - 1) / WAVES;           // every wavefront issues this many per step (4)
   static constexpr int WBYTES = WPIECES * 1024;
   static constexpr int STAGE = WBYTES + 8192 * HV;
   static constexpr int LDS = 3 * STAGE;
@@ -491,35 +493,34 @@ template <int WT, int HV> struct TgxGeom {
 //      height; the last may be shorter): chunk k owns the partial slots k*spc .. k*spc+spc-1, and no label range crosses
 //      a chunk boundary, so that each chunk's sum can be rounded by itself.
 template <int WT, int HV>
-__global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
+__global__ __launch_bounds__(256 * HV) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
                                                           const unsigned short* gbl, size_t g_half, floatx4* partial, size_t part_half) {
   typedef TgxGeom<WT, HV> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
   const unsigned lds0 = (unsigned)(size_t)lds;
   const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
+  const int fw = wv & 3, hw = wv >> 2;   // this wavefront's 48 features of the quarter, its batch half
   // The four workgroups of a label range read the same G^T: they sit on one XCD (workgroups go to the XCDs round robin),
   // eight apart in launch order, so that three of the four reads are served by that XCD's L2.
   const int fb = ((int)blockIdx.x >> 3) & 3, split = ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7);
   const int ck = split / spc, lbeg = ck * cs + (split - ck * spc) * range;
   const int cend = min((ck + 1) * cs, bound);   // bound: the launch's rows rounded up to a tile
   if (lbeg >= cend) return;                     // the grid is rounded up to eight ranges; a short last chunk has fewer
-  floatx4 acc[HV][8][3];
+  floatx4 acc[8][3];
 #pragma unroll
-  for (int hv = 0; hv < HV; hv++)
+  for (int mb = 0; mb < 8; mb++)
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++)
-#pragma unroll
-      for (int nn = 0; nn < 3; nn++) acc[hv][mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lend = min(lbeg + range, cend);
   const int nsteps = (lend - lbeg + 31) >> 5;
-  // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv+4, ...; indices past the last piece repeat it),
+  // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv + WAVES, ...; indices past the last piece repeat it),
   // so that "all but the newest PER_WAVE" means the step before has landed.  Steps past the end repeat the last one.
   auto issue_step = [&](int st, int stage) {
     const int l0 = lbeg + 32 * min(st, nsteps - 1);
 #pragma unroll
     for (int j = 0; j < G::PER_WAVE; j++) {
-      const int piece = min(wv + 4 * j, G::PIECES - 1);
+      const int piece = min(wv + G::WAVES * j, G::PIECES - 1);
       if (piece < G::WPIECES) {
         const int ch = min(piece * 64 + lane, 32 * G::SLOTS - 1), row = ch / G::SLOTS, c16 = min(ch - row * G::SLOTS, G::SLOTS - 2);
         const int lr = min(l0 + row, rows - 1);   // rows past the end re-read a valid one (their G is zero)
@@ -545,22 +546,17 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
     const __attribute__((address_space(3))) unsigned char* gt = wt + G::WBYTES;
     bf16x8 ga[8];
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + (mb * 64 + lane) * 16);
-    bf16x8 gh[HV == 2 ? 8 : 1];
-    if (HV == 2) {
-#pragma unroll
-      for (int mb = 0; mb < 8; mb++) gh[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + 8192 + (mb * 64 + lane) * 16);
-    }
+    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + hw * 8192 + (mb * 64 + lane) * 16);
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
       if (WT == W_BF16) {
-        const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * G::STRIDE + (48 * wv + 16 * nn + 4 * (l16 & 3)) * 2);
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * G::STRIDE + (48 * fw + 16 * nn + 4 * (l16 & 3)) * 2);
         tshortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off));
         tshortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off + 4 * G::STRIDE));
         wb[nn] = __builtin_bit_cast(bf16x8, tshortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
       } else {
-        const unsigned off = (unsigned)((8 * kg + (l16 >> 1)) * G::STRIDE + 48 * wv + 16 * nn + (l16 & 1) * 8);
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 1)) * G::STRIDE + 48 * fw + 16 * nn + (l16 & 1) * 8);
         const intx2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(wt + off));
         wb[nn] = t_fp8x8_to_bf16x8(raw);
       }
@@ -568,26 +564,16 @@ __global__ __launch_bounds__(256) void tiled_gradx_kernel(const void* w, int row
 #pragma unroll
     for (int mb = 0; mb < 8; mb++)
 #pragma unroll
-      for (int nn = 0; nn < 3; nn++) acc[0][mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[0][mb][nn], 0, 0, 0);
-    if (HV == 2) {
-#pragma unroll
-      for (int mb = 0; mb < 8; mb++)
-#pragma unroll
-        for (int nn = 0; nn < 3; nn++)
-          acc[HV - 1][mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gh[mb], wb[nn], acc[HV - 1][mb][nn], 0, 0, 0);
-    }
+      for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
     stage = stage == 2 ? 0 : stage + 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end still target LDS
-  // acc[mb][nn][e] = C[batch 16mb + 4kg + e][feature f0 + 16nn + l16]
+  // acc[mb][nn][e] = C[batch 128hw + 16mb + 4kg + e][feature 192fb + 48fw + 16nn + l16]
+  floatx4* dst = partial + (size_t)hw * part_half + ((size_t)split * 4 + fb) * 24 * 256;
 #pragma unroll
-  for (int hv = 0; hv < HV; hv++) {
-    floatx4* dst = partial + (size_t)hv * part_half + ((size_t)split * 4 + fb) * 24 * 256;
+  for (int mb = 0; mb < 8; mb++)
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++)
-#pragma unroll
-      for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + tid] = acc[hv][mb][nn];
-  }
+    for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + fw * 64 + lane] = acc[mb][nn];
 }
 
 // sum of the partials of one chunk and batch half in a fixed order; bf16 weights: the chunk's contribution is rounded to
