@@ -584,10 +584,10 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       const unsigned short* gsrc = gbl + h0 * g_half;
       floatx4* pdst = partial + h0 * part_half;
       if (weight_type == W_BF16) {
-        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<ggrid, 256, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<ggrid, 512, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
         else tiled_gradx_kernel<W_BF16, 2><<<ggrid, 512, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       } else {
-        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<ggrid, 256, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<ggrid, 512, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
         else tiled_gradx_kernel<W_E4M3, 2><<<ggrid, 512, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       }
     }

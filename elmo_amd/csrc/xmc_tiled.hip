@@ -474,16 +474,18 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
 //      memory path handles few cache lines per clock, and register loads in operand order touched four times as many.
 //      The W operand comes back transposed (ds_read_b64_tr_b8 + exact fp8->bf16, or ds_read_b64_tr_b16).
 //      With two batch halves (HV = 2) one pass over W serves both: the step's G^T of either half is staged, and the
-//      workgroup has eight wavefronts, four per half (two per SIMD: one's LDS reads and conversions run under the
-//      other's matrix instructions; with both halves' accumulators in one wavefront a SIMD had a single wavefront).
+//      workgroup's eight wavefronts are four per half; with one half they are four per four batch blocks (two wavefronts
+//      per SIMD either way: one's LDS reads and conversions run under the other's matrix instructions).
 template <int WT, int HV> struct TgxGeom {
   static constexpr int ROWB = WT == W_BF16 ? 384 : 192;                  // bytes of this workgroup's features in one row
   static constexpr int STRIDE = ROWB + 16;                                // LDS row stride
   static constexpr int SLOTS = STRIDE / 16;                               // 16-byte slots per LDS row, the last one padding
   static constexpr int WPIECES = (32 * SLOTS + 63) / 64;                  // wave-wide loads of the W slice (7 or 13)
   static constexpr int PIECES = WPIECES + 8 * HV;                         // ... and of G^T (8 per batch half)
-  static constexpr int WAVES = 4 * HV;                                    // four wavefronts (48 features each) per batch half
-  static constexpr int PER_WAVE = (PIECES + WAVES - 1) / WAVES;           // every wavefront issues this many per step (4)
+  static constexpr int WAVES = 8;                                         // four wavefronts (48 features each) per batch half or,
+                                                                          // with one half, per four of its eight batch blocks
+  static constexpr int NMB = 4 * HV;                                      // batch blocks of 16 rows per wavefront
+  static constexpr int PER_WAVE = (PIECES + WAVES - 1) / WAVES;           // every wavefront issues this many per step (2 - 4)
   static constexpr int WBYTES = WPIECES * 1024;
   static constexpr int STAGE = WBYTES + 8192 * HV;
   static constexpr int LDS = 3 * STAGE;
@@ -493,23 +495,24 @@ template <int WT, int HV> struct TgxGeom {
 //      height; the last may be shorter): chunk k owns the partial slots k*spc .. k*spc+spc-1, and no label range crosses
 //      a chunk boundary, so that each chunk's sum can be rounded by itself.
 template <int WT, int HV>
-__global__ __launch_bounds__(256 * HV) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
+__global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
                                                           const unsigned short* gbl, size_t g_half, floatx4* partial, size_t part_half) {
   typedef TgxGeom<WT, HV> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
   const unsigned lds0 = (unsigned)(size_t)lds;
   const int tid = threadIdx.x, wv = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
-  const int fw = wv & 3, hw = wv >> 2;   // this wavefront's 48 features of the quarter, its batch half
+  // this wavefront's 48 features of the quarter; its batch half, or with one half its four batch blocks
+  const int fw = wv & 3, hw = HV == 2 ? wv >> 2 : 0, mb0 = HV == 2 ? 0 : 4 * (wv >> 2);
   // The four workgroups of a label range read the same G^T: they sit on one XCD (workgroups go to the XCDs round robin),
   // eight apart in launch order, so that three of the four reads are served by that XCD's L2.
   const int fb = ((int)blockIdx.x >> 3) & 3, split = ((int)blockIdx.x >> 5) * 8 + ((int)blockIdx.x & 7);
   const int ck = split / spc, lbeg = ck * cs + (split - ck * spc) * range;
   const int cend = min((ck + 1) * cs, bound);   // bound: the launch's rows rounded up to a tile
   if (lbeg >= cend) return;                     // the grid is rounded up to eight ranges; a short last chunk has fewer
-  floatx4 acc[8][3];
+  floatx4 acc[G::NMB][3];
 #pragma unroll
-  for (int mb = 0; mb < 8; mb++)
+  for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lend = min(lbeg + range, cend);
@@ -544,9 +547,10 @@ __global__ __launch_bounds__(256 * HV) void tiled_gradx_kernel(const void* w, in
     issue_step(st + 2, stage == 0 ? 2 : stage - 1);
     const __attribute__((address_space(3))) unsigned char* wt = lds + stage * G::STAGE;
     const __attribute__((address_space(3))) unsigned char* gt = wt + G::WBYTES;
-    bf16x8 ga[8];
+    bf16x8 ga[G::NMB];
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++) ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + hw * 8192 + (mb * 64 + lane) * 16);
+    for (int mb = 0; mb < G::NMB; mb++)
+      ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + hw * 8192 + ((mb0 + mb) * 64 + lane) * 16);
     bf16x8 wb[3];
 #pragma unroll
     for (int nn = 0; nn < 3; nn++) {
@@ -562,18 +566,18 @@ __global__ __launch_bounds__(256 * HV) void tiled_gradx_kernel(const void* w, in
       }
     }
 #pragma unroll
-    for (int mb = 0; mb < 8; mb++)
+    for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
       for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
     stage = stage == 2 ? 0 : stage + 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end still target LDS
-  // acc[mb][nn][e] = C[batch 128hw + 16mb + 4kg + e][feature 192fb + 48fw + 16nn + l16]
+  // acc[mb][nn][e] = C[batch 128hw + 16(mb0 + mb) + 4kg + e][feature 192fb + 48fw + 16nn + l16]
   floatx4* dst = partial + (size_t)hw * part_half + ((size_t)split * 4 + fb) * 24 * 256;
 #pragma unroll
-  for (int mb = 0; mb < 8; mb++)
+  for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + fw * 64 + lane] = acc[mb][nn];
+    for (int nn = 0; nn < 3; nn++) dst[((mb0 + mb) * 3 + nn) * 256 + fw * 64 + lane] = acc[mb][nn];
 }
 
 // sum of the partials of one chunk and batch half in a fixed order; bf16 weights: the chunk's contribution is rounded to
