@@ -103,3 +103,54 @@ def test_sampled_rows_match_oracle_after_a_real_step(gpu, big):
     d = H.e4m3_ulp_distance(got, ref_codes[0])
     assert d.max() <= 1 and np.mean(d != 0) < 2e-3
     assert np.mean(got != w_old) > 0.3                       # the step really changed the weights
+
+
+def test_batch_256_at_the_chunk_size_of_the_largest_workload(gpu):
+    """True FP8 with 256 batch rows on chunks of 262,144 rows (the chunk size of the 8.6 M-label workload, four chunks
+    here): the one-pass FP8 logits, the eight-wavefront grad_X and the feature-split update at their real launch shapes.
+    lr = 0 leaves the weights alone; after a real step sampled rows equal the oracle's; grad_X equals fp64 library
+    GEMMs on the same device."""
+    import torch
+    from elmo_amd import ops
+    nc, rows, batch, L = 4, 262144, 256, 4 * 262144 - 37
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.02).to(torch.float8_e4m3fn) for _ in range(nc)]
+    x_np = synth.make_x(batch, 768, 5)
+    labels_np = synth.make_labels(batch, L, 8.0, 1.1, 5)
+    x = torch.from_numpy(x_np).to(gpu).to(torch.bfloat16)
+    labels = torch.from_numpy(labels_np).to(gpu)
+    ws = ops.alloc_tiled_workspace(nc, rows, gpu, batch)
+    kw = dict(round_mode="rtn", workspace=ws, quantize_x=True, saturate=True, want_f32=True)
+    before = [c.view(torch.uint8).clone() for c in chunks]
+    g, gf = ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.0, **kw)
+    for a, c in zip(before, chunks):
+        b = c.view(torch.uint8)
+        assert bool(((a == b) | (((a | b) & 0x7F) == 0)).all())
+    xq = x.to(torch.float8_e4m3fn).float()
+    ref = torch.zeros(batch, 768, device=gpu, dtype=torch.float64)
+    lab = labels.long()
+    for c, wc in enumerate(chunks):
+        w = wc.float()
+        z = (w @ xq.t()).to(torch.bfloat16).float()
+        s = torch.sigmoid(z).to(torch.bfloat16)
+        sel = (lab[:, 1] >= c * rows) & (lab[:, 1] < (c + 1) * rows)
+        s[lab[sel, 1] - c * rows, lab[sel, 0]] -= 1.0
+        ref += (s.double().t() @ w.double())
+        del w, z, s
+    ref = ref.float()
+    assert (gf - ref).abs().max().item() <= 2e-3 * ref.abs().max().item()
+    assert torch.equal(g.view(torch.int16), gf.to(torch.bfloat16).view(torch.int16))
+    # a real step: sampled rows (tile and chunk boundaries, the head labels, random ones) against the oracle
+    rng = np.random.default_rng(1)
+    pos_rows = np.unique(labels_np[:, 1])
+    sample = np.unique(np.concatenate([np.arange(0, 130), pos_rows[:300], [rows - 1, rows, rows + 1, 3 * rows - 1, 3 * rows, nc * rows - 1],
+                                       rng.integers(0, nc * rows, 500)]))
+    w_old = np.stack([chunks[r // rows][r % rows].view(torch.uint8).cpu().numpy().copy() for r in sample])
+    ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.05, **kw)
+    remap = {int(r): i for i, r in enumerate(sample)}
+    lab_s = np.array([(b, remap[int(l)]) for b, l in labels_np if int(l) in remap], dtype=np.int32).reshape(-1, 2)
+    ref_codes, _, _ = O.fp8_step([w_old], x_np, lab_s, 0.05, sr_mode="rtn")
+    got = np.stack([chunks[r // rows][r % rows].view(torch.uint8).cpu().numpy() for r in sample])
+    d = H.e4m3_ulp_distance(got, ref_codes[0])
+    assert d.max() <= 1 and np.mean(d != 0) < 2e-3
+    assert np.mean(got != w_old) > 0.3
