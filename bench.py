@@ -128,8 +128,9 @@ def bench_tiled(args, cfg):
     grad = torch.empty(cfg.batch, cfg.dim, dtype=torch.bfloat16, device=dev)
     true_fp8 = not bf16 and "simfp8" not in cfg.name
     rng = np.random.default_rng(cfg.seed)
-    # the reference's Philox recipe where it is the only stochastic mode (bf16 weights, simulated FP8)
-    mode = args.round if true_fp8 or args.round == "rtn" else "sr_philox"
+    # bf16 weights and simulated FP8 round with the reference's Philox recipe unless another mode is asked for by name
+    # (simulated FP8 has no fast mode: its cast goes through bf16 and torch)
+    mode = args.round if true_fp8 or args.round == "rtn" or (bf16 and args.round_given) else "sr_philox"
 
     def one_step():
         ops.tiled_step(views, rows, wtype, x, labels, cfg.lr, seeds=rng.integers(0, 1_000_000, size=len(views)),
@@ -281,6 +282,7 @@ def main():
     from elmo_amd import _lib, ops, synth
 
     cfg = synth.CONFIGS[args.config]
+    args.round_given = args.round is not None
     if args.round is None:   # the first workload is defined with round-to-nearest, the others with stochastic rounding
         args.round = "rtn" if args.config == "cfg1_bf16_131k" else "sr_fast"
     if cfg.batch > ops.MAX_BATCH_TILED:

@@ -57,7 +57,7 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
     // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
 #define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
-    XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false);
+    XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_FAST, false);
     XMC_UPD_ATTR(W_E4M3, ROUND_RTN, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, false);
     XMC_UPD_ATTR(W_E4M3, ROUND_RTN, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, true);
 #undef XMC_UPD_ATTR
@@ -479,7 +479,6 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1 || nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
   if (weight_type != W_E4M3 && weight_type != W_BF16) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX && round_mode != XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
-  if (round_mode == XMC_ROUND_SR_FAST && weight_type != W_E4M3) return XMC_ERR_MODE;   // the converter rounds to e4m3
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
   for (int c = 0; c < num_chunks; c++) {
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
@@ -618,6 +617,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
 #undef XMC_LAUNCH_UPDATE2
     } else if (weight_type == W_BF16) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_RTN, false);
+      else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_SR_FAST, false);
       else XMC_LAUNCH_UPDATE_H(W_BF16, ROUND_SR_PHILOX, false);
     } else if (with_head) {
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE_H(W_E4M3, ROUND_RTN, true);

@@ -669,8 +669,22 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
     }
   }
   if (WT == W_BF16) {
-    wout[0] = (unsigned)bf16_bits(t[0]) | ((unsigned)bf16_bits(t[1]) << 16);
-    wout[1] = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
+    if (MODE == ROUND_SR_FAST) {
+      // the converter adds the upper half of the random word to the fp32 pattern and drops the lower 16 bits; the words
+      // are those of the FP8 fast mode (one counter hash per four weights)
+      typedef __bf16 t_bf16x2 __attribute__((ext_vector_type(2)));
+      const unsigned hsh = fast_mix(fidx, seed);
+      t_bf16x2 lo = {}, hi = {};
+      lo = __builtin_amdgcn_cvt_sr_bf16_f32(lo, t[0], fast_word(hsh, 0), false);
+      lo = __builtin_amdgcn_cvt_sr_bf16_f32(lo, t[1], fast_word(hsh, 1), true);
+      hi = __builtin_amdgcn_cvt_sr_bf16_f32(hi, t[2], fast_word(hsh, 2), false);
+      hi = __builtin_amdgcn_cvt_sr_bf16_f32(hi, t[3], fast_word(hsh, 3), true);
+      wout[0] = __builtin_bit_cast(unsigned, lo);
+      wout[1] = __builtin_bit_cast(unsigned, hi);
+    } else {
+      wout[0] = (unsigned)bf16_bits(t[0]) | ((unsigned)bf16_bits(t[1]) << 16);
+      wout[1] = (unsigned)bf16_bits(t[2]) | ((unsigned)bf16_bits(t[3]) << 16);
+    }
   } else {
     if (saturate) {
 #pragma unroll

@@ -228,8 +228,8 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
         ktype = 1 if kahan.dtype == torch.bfloat16 else 2
     assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
     assert labels.dim() == 2 and labels.shape[1] == 2
-    assert round_mode in ("rtn", "sr_philox") or (round_mode == "sr_fast" and weight_type == "e4m3"), \
-        "the tiled path rounds to nearest, with the reference's Philox recipe or (e4m3 weights) with the fast hardware mode"
+    assert round_mode in ("rtn", "sr_philox", "sr_fast"), \
+        "the tiled path rounds to nearest, with the reference's Philox recipe or with the fast hardware mode"
     wdt = (torch.bfloat16,) if weight_type == "bf16" else (torch.float8_e4m3fn, torch.uint8)
     nc = len(chunk_views)
     arr = (ctypes.c_void_p * nc)()

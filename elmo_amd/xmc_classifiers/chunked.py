@@ -15,7 +15,9 @@ fp32 / fp16 weights (precision mode 'purefp', model.xmc.dtype float16/float32) t
 GPU) and elementwise torch operations in the weight's type, with weight decay: A += wd*W; W += -lr*A.  It is restated
 here operation by operation, on the GPU, for any batch size; momentum stays unused as in the reference.
 
-Optional, not in the reference: training.xmc.rounding = "sr_philox" (default: the reference's Philox recipe) | "rtn".
+Optional, not in the reference: training.xmc.rounding = "sr_philox" (default: the reference's Philox recipe) | "rtn" |
+"sr_fast" (the hardware's stochastic conversion to bf16 with a counter hash: unbiased, not the reference's random stream,
+and not bound by the 48 vector instructions per weight of the Philox recipe).
 """
 import torch
 from torch import nn
@@ -65,7 +67,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
             self.momentum_buff = torch.zeros(self.num_labels, features, dtype=self._dtype, device=self.device)
 
         self.rounding = _opt(cfg.training.xmc, "rounding", "sr_philox")
-        assert self.rounding in ("sr_philox", "rtn")
+        assert self.rounding in ("sr_philox", "rtn", "sr_fast")
         self.wd = float(_opt(cfg.training.xmc, "wd", 0.0))      # used by the fp32 / fp16 branch only (chunked.py:123)
         self.grad_input = torch.zeros(cfg.data.batch_size, features, dtype=self._dtype, device=self.device)
         self.dummy = torch.zeros(1, dtype=self._dtype, device=self.device)

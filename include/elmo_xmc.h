@@ -39,7 +39,7 @@ enum {
 enum {
   XMC_ROUND_RTN = 0,        /* round to nearest even, saturating at +-448 */
   XMC_ROUND_SR_PHILOX = 1,  /* the reference bit recipe: Philox-4x32-10 word per element, add 20 bits, mask, cast */
-  XMC_ROUND_SR_FAST = 2     /* unbiased stochastic rounding on the e4m3 grid (hardware converter, counter hash) */
+  XMC_ROUND_SR_FAST = 2     /* unbiased stochastic rounding on the e4m3 (or bf16) grid (hardware converter, counter hash) */
 };
 
 int xmc_version(void);
@@ -169,8 +169,9 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
- *   round_mode       XMC_ROUND_RTN, XMC_ROUND_SR_PHILOX, or (e4m3 weights only) XMC_ROUND_SR_FAST with the random words of
- *                    xmc_fp8_step's mode of that name; batch: 1..512, any value (processed in one, two or four halves of 128 rows)
+ *   round_mode       XMC_ROUND_RTN, XMC_ROUND_SR_PHILOX, or XMC_ROUND_SR_FAST with the random words of xmc_fp8_step's
+ *                    mode of that name (bf16 weights: the hardware converter to bf16, which adds the upper 16 bits of the
+ *                    word to the fp32 pattern); batch: 1..512, any value (processed in one, two or four halves of 128 rows)
  *   quantize_x       e4m3 weights: 0 = logits from the un-quantised X (simulated FP8), 1 = from e4m3(X) (true FP8, :101)
  *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
  *   kahan, kahan_type, num_head

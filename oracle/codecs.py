@@ -219,6 +219,16 @@ def sr_e4m3_exact(t, rand32):
     return e4m3_encode(np.copysign(v, t), saturate=True)
 
 
+def sr_bf16_fast(t, rand32):
+    """fp32 -> bf16 value as the hardware converter of this build's fast mode rounds (v_cvt_sr_bf16_f32): the upper 16 bits
+    of the random word are added to the fp32 bit pattern and the lower 16 bits dropped - round up with probability equal
+    to the dropped fraction.  Not part of the reference (whose recipe adds the low 16 bits of a Philox word, sr_add_mask)."""
+    t = np.ascontiguousarray(t, dtype=np.float32)
+    u = t.view(np.uint32).astype(np.uint64) + (np.asarray(rand32).astype(np.uint64) >> np.uint64(16))
+    u = (u & np.uint64(0xFFFF0000)).astype(np.uint32)
+    return u.view(np.float32).reshape(t.shape)
+
+
 # --------------------------------------------------------------------------- this build's fast SR random words
 def fast_sr_words(seed, global_rows, cols, features=768):
     """Random word per weight of the fast stochastic-rounding mode (not part of the reference): one 32-bit mix per

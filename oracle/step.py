@@ -202,6 +202,7 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
     w_bf16 : fp32 array [L, d] holding bf16 values (single tensor, chunk views of ceil(L/nc) rows, last short)
     sr_mode: "rtn"        W' = bf16(f32(W) - lr*f32(A))
              "reference"  W' = SR16(f32(W) - f32(A)*lr; philox(seed_c, flat idx in chunk))  (stochastic_rounding_kernel.py:80-89)
+             "fast"       the same T rounded by sr_bf16_fast with the counter-hash words of the FP8 fast mode (not in the reference)
     Weight decay is ignored exactly as the bf16 path of the reference ignores it (:91-99).
     Returns (new_w [L,d] bf16-valued fp32, gx_fp32 [B,d], grad_input bf16-valued fp32[, loss with return_loss]).
     """
@@ -236,6 +237,12 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
             t = (w64 - a.astype(np.float64) * float(lr32)).astype(np.float32)   # stochastic_rounding_kernel.py:81 (fma)
             offs = np.arange((hi - lo) * d, dtype=np.int64).reshape(hi - lo, d)
             nw = C.sr_bf16_reference(t, seeds[c], offs)
+        elif sr_mode == "fast":
+            # this build's own mode: hardware stochastic rounding fed with the counter-hash words of the FP8 fast mode
+            t = (w64 - a.astype(np.float64) * float(lr32)).astype(np.float32)
+            grow = np.arange(lo, hi, dtype=np.int64)[:, None] + np.zeros((1, d), dtype=np.int64)
+            cols = np.zeros((hi - lo, 1), dtype=np.int64) + np.arange(d, dtype=np.int64)[None, :]
+            nw = C.sr_bf16_fast(t, C.fast_sr_words(seeds[c], grow, cols, d))
         else:
             raise ValueError(sr_mode)
         new_w[lo:hi] = nw

@@ -221,3 +221,20 @@ def test_fast_rounding_words_look_uniform_and_independent():
     w2 = C.fast_sr_words(12346, np.broadcast_to(rows, (4096, 768)), np.broadcast_to(cols, (4096, 768)))
     u2 = (w2 >> np.uint32(12)).astype(np.float64) / float(1 << 20)
     assert abs(corr(u, u2)) < 5.0 / np.sqrt(n)                                                      # next seed
+
+
+@pytest.mark.parametrize("value", [1.00390625 * 1.3, -7.77, 3.3e-5, 1.0])
+def test_sr_bf16_fast_probability_equals_dropped_fraction_exhaustively(value):
+    """The fast mode's rounding to bf16 over all 2^16 values of the upper half of the random word (the lower half must not
+    matter): floor or ceil in magnitude, ceil exactly `dropped bits` times out of 2^16, a bf16 value unchanged."""
+    t = np.full(1 << 16, value, dtype=np.float32)
+    hi = np.arange(1 << 16, dtype=np.uint64) << np.uint64(16)
+    out = C.sr_bf16_fast(t, hi | np.uint64(0xABCD))
+    assert np.array_equal(out, C.sr_bf16_fast(t, hi))
+    bits = int(t.view(np.uint32)[0])
+    lo_f = np.array([bits & 0xFFFF0000], dtype=np.uint32).view(np.float32)[0]
+    hi_f = np.array([(bits & 0xFFFF0000) + 0x10000], dtype=np.uint32).view(np.float32)[0]
+    assert set(np.unique(out)) <= {lo_f, hi_f}
+    assert int((out == hi_f).sum()) == (bits & 0xFFFF) or (bits & 0xFFFF) == 0
+    # the reference's recipe with the same 16 bits in the low half gives the same values (it adds the LOW 16 bits)
+    assert np.array_equal(out, C.sr_add_mask(t, hi >> np.uint64(16), 16))

@@ -374,10 +374,10 @@ def test_true_fp8_fast_rounding_on_the_three_kernel_path(gpu):
         assert d.max() <= 1
         mism += int((d != 0).sum()); total += d.size
     assert mism / total < 2e-3, (mism, total)
-    # bf16 weights have no such mode
+    # an unknown mode is refused before anything is launched
     w = torch_bf16_weights(gpu, 64)
     with pytest.raises(AssertionError):
-        ops.tiled_step([w], 64, "bf16", x[:16], labels[:0], 0.05, seeds=[1], round_mode="sr_fast")
+        ops.tiled_step([w], 64, "bf16", x[:16], labels[:0], 0.05, seeds=[1], round_mode="sr_exact")
 
     case = H.make_case(nc, rows, 64, 65)
     c1, x1, l1 = H.to_device_case(case, gpu)
@@ -551,3 +551,51 @@ def test_e4m3_chunks_in_one_allocation_take_one_launch(gpu, mode, quant):
     assert torch.equal(torch.cat(chunks).view(torch.uint8), whole.view(torch.uint8))
     assert torch.equal(g0.view(torch.int16), g1.view(torch.int16))
     assert torch.allclose(gf0, gf1, rtol=0, atol=1e-6 * float(gf0.abs().max()))
+
+
+def test_bf16_layer_fast_stochastic_rounding(gpu):
+    """The bf16 layer with this build's fast mode (hardware conversion to bf16, counter-hash words): equal to the oracle
+    wherever the fp32 value it rounds is (as for the Philox recipe), different from round-to-nearest, seed-dependent,
+    and unbiased: over more than a million weights the mean error against the exact update is below 1e-3 of the mean
+    |delta w| (round-to-nearest of such small updates is not)."""
+    L, nc, batch = 2048, 2, 64
+    x, w, labels = bf16_case(L, batch, 43, pos_mean=20.0)
+    seeds = [4242, 77]
+    new, gf, gb = run_bf16(x, w, labels, nc, gpu, "sr_fast", seeds, lr=0.5)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.5, nc, seeds=seeds, sr_mode="fast")
+    check_bf16_weights(new, ref_w, w, x, lr=0.5)
+    check_gx(gf, gb, ref_gx, tol=4e-3)
+    rtn_w, _, _ = O.bf16_step(w, x, labels, 0.5, nc, sr_mode="rtn")
+    assert (new != rtn_w).mean() > 0.2
+    new2, _, _ = run_bf16(x, w, labels, nc, gpu, "sr_fast", [1, 2], lr=0.5)
+    assert (new2 != new).mean() > 0.1
+    # unbiasedness against the exact (fp64) update t = w - lr * bf16(A)
+    parts = O.bf16_step(w, x, labels, 0.5, nc, sr_mode="rtn", return_parts=True)[-1]
+    t = np.concatenate([p["t"] for p in parts]).astype(np.float64)
+    assert t.size > 10 ** 6
+    dw = np.abs(t - w).mean()
+    assert abs((new.astype(np.float64) - t).mean()) <= 1e-3 * dw
+
+
+def test_chunked_module_with_the_fast_rounding(gpu):
+    """XMCBCECHUNKEDLayer with training.xmc.rounding = "sr_fast": the step equals the oracle's with the seeds the module
+    drew from the global CPU generator (one per chunk, as the reference draws them, chunked.py:126)."""
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked import XMCBCECHUNKEDLayer
+    cfg = make_cfg("cuda:0", 1000, 3, rounding="sr_fast")
+    cfg.model.xmc.dtype = "bfloat16"
+    torch.manual_seed(3)
+    xfc = XMCBCECHUNKEDLayer(cfg)
+    emb = torch.randn(32, 768, device=gpu, dtype=torch.bfloat16)
+    labels = torch.tensor([[0, 3], [1, 999], [5, 17], [31, 500]], dtype=torch.int32, device=gpu)
+    w0 = xfc.xfc_weight.float().cpu().numpy()
+    torch.manual_seed(11)
+    seeds = [torch.randint(0, 1000000, (1,)).item() for _ in range(3)]
+    torch.manual_seed(11)
+    xfc.xfc_forward_backward(emb, labels, [0.5], skip_loss=True)
+    x_np = emb.float().cpu().numpy()
+    ref_w, _, _ = O.bf16_step(w0, x_np, labels.cpu().numpy(), 0.5, 3, seeds=seeds, sr_mode="fast")
+    check_bf16_weights(xfc.xfc_weight.float().cpu().numpy(), ref_w, w0, x_np, lr=0.5)
+    rtn_w, _, _ = O.bf16_step(w0, x_np, labels.cpu().numpy(), 0.5, 3, sr_mode="rtn")
+    assert (xfc.xfc_weight.float().cpu().numpy() != rtn_w).mean() > 0.1
