@@ -233,9 +233,10 @@ def bench_inference(args, cfg):
     achieved = algo_bytes / (dev_ms * 1e-3) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath) and not topk:
+    if os.path.exists(tpath) and not chunkwise:   # from the profile summaries, not measured in this run
         with open(tpath) as f:
-            traffic = json.load(f).get(f"fp8_forward_kernel:{cfg.name}:forward")
+            traffic = json.load(f).get(f"fp8_forward_select_kernel:{cfg.name}:forward_topk" if topk else
+                                       f"fp8_forward_kernel:{cfg.name}:forward")
     print(json.dumps({
         "metric": "XMC classifier inference calls/sec, " + ("top-100 per row without the dense logits" if topk else "dense logits"),
         "value": args.steps / elapsed, "unit": "calls/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
