@@ -3,6 +3,7 @@
 #include "../../include/elmo_xmc.h"
 #include "xmc_fp8_forward.hip"
 #include "xmc_fp8_quad.hip"
+#include "xmc_fp8_role.hip"
 #include "xmc_tiled.hip"
 #include "xmc_topk.hip"
 #include "xmc_dropout.hip"
@@ -40,6 +41,9 @@ DeviceInfo device_info() {
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
     (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
     (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
@@ -223,15 +227,28 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
         (unsigned short*)(ws + WS_XT));
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
-    switch (round_mode) {
-      case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
-      case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
-      default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+    static const bool old_kernel = getenv("XMC_STEP_KERNEL") && !__builtin_strcmp(getenv("XMC_STEP_KERNEL"), "quad");
+    if (old_kernel) {
+      switch (round_mode) {
+        case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+        case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+        default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
+      }
+    } else {
+      switch (round_mode) {
+        case XMC_ROUND_RTN: fp8_step_role_kernel<ROUND_RTN><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+        case XMC_ROUND_SR_PHILOX: fp8_step_role_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+        default: fp8_step_role_kernel<ROUND_SR_FAST><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+      }
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
-    reduce_gx_quad_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
-                                                 (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
+    if (old_kernel)
+      reduce_gx_quad_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+                                                   (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
+    else
+      reduce_gx_role_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+                                                   (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
   }
   return launch_status();
 }

@@ -28,18 +28,22 @@ constexpr int MAX_WG = 256;                                   // workgroups of t
 constexpr size_t WS_XQ = 0;                                   // FP8 logits operands   BP*D
 constexpr size_t WS_XT = WS_XQ + (size_t)BP * D;              // bf16 grad_W operands  BP*D*2
 constexpr size_t WS_KEYS = WS_XT + (size_t)BP * D * 2;        // sorted positive keys  MAX_POS*4
-constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // 1024 ints: counters, XCC ids, error word (below)
-constexpr size_t WS_PARTIAL = WS_FLAGS + 4096;                // MAX_WG * 12 * 512 * 16 bytes of grad_X partials
+constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // 2048 ints: counters, XCC ids, error words (below)
+constexpr size_t WS_PARTIAL = WS_FLAGS + 8192;                // MAX_WG * 12 * 512 * 16 bytes of grad_X partials
 constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 12 * 512 * 16;     // G exchange ring: 64 quads x 8 slots x 20 KiB
 constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 8 * 20480;   // tile_ptr[num_tiles + 1], then the tile descriptors
 
-// Layout of the 1024 ints at WS_FLAGS (cleared at the start of every step):
-//   [0, 256)              tiles-published / tiles-loaded counters of the persistent step kernels
-//   [QF_XCC, QF_XCC+256)  XCC id every workgroup of the quad kernel found itself on
+// Layout of the 2048 ints at WS_FLAGS (all but the last cleared at the start of every step):
+//   [0, 1024)             tiles-published counters of the persistent step kernel: sixteen per quad
+//   [QF_XCC, QF_XCC+256)  XCC id every workgroup of the step kernel found itself on
 //   [QF_ERR]              error word: bit 0 = a bounded wait expired, bit 1 = the workgroups of a quad were not placed on
 //                         one XCD (their exchange of G through that XCD's L2 is then not coherent)
-constexpr int QF_XCC = 512;
-constexpr int QF_ERR = 1020;
+//   [QF_STICKY]           the error words of all steps since the caller last cleared it, OR-ed together by the step's
+//                         last kernel; no kernel ever clears it
+constexpr int QF_WORDS = 2048;
+constexpr int QF_XCC = 1024;
+constexpr int QF_ERR = 2044;
+constexpr int QF_STICKY = 2047;
 
 // The quad kernel assumes that workgroup g runs on XCD g % 8, and builds quads of four workgroups with equal g % 8:
 // member m of quad q is workgroup ((q / 8) * 4 + m) * 8 + q % 8.

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
   extern __shared__ unsigned sk[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   if (blockIdx.x == 0 && flags)
-    for (int i = tid; i < 1024; i += 256) flags[i] = 0;
+    for (int i = tid; i < QF_STICKY; i += 256) flags[i] = 0;
   if (n_pad == 0) return;
   // eight (row, label) pairs per thread in flight at a time: the loads miss every cache
   const int2* coo2 = (const int2*)coo;
