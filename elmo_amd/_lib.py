@@ -72,6 +72,7 @@ def load():
     lib.xmc_dropout_quantize.restype = i32
     lib.xmc_dropout_quantize.argtypes = [vp, i32, i32, i32, f32, ctypes.c_ulonglong, vp, vp]
     lib.xmc_step_error_offset.restype = sz
+    lib.xmc_step_sticky_error_offset.restype = sz
     lib.xmc_step_workgroups.restype = i32
     lib.xmc_step_xcc_ids.restype = i32
     lib.xmc_step_xcc_ids.argtypes = [vp, ctypes.POINTER(ctypes.c_int32), i32, vp]

@@ -38,9 +38,6 @@ DeviceInfo device_info() {
     cached[dev].scratch_ptr = (cached[dev].ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess)
                                   ? (unsigned char*)sp : nullptr;
     // opt in to the full 160 KiB of LDS once per device
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_quad_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, QLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
     (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
@@ -216,7 +213,10 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.zscale = scale_w * scale_x;
     p.lr_eff = lr / scale_w;
     p.batch = batch;
-    const int qgrid = grid / 32 * 32;   // whole quads on every XCD
+    int qgrid = grid / 32 * 32;   // whole quads on every XCD
+#ifdef XMC_DEV_GRID
+    if (getenv("XMC_STEP_GRID")) qgrid = atoi(getenv("XMC_STEP_GRID"));   // working builds only
+#endif
     if (qgrid < 32) return XMC_ERR_DEVICE;
     p.nquads = qgrid >> 2;
     p.kmax = (num_tiles + p.nquads - 1) / p.nquads;
@@ -227,28 +227,15 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
         (unsigned short*)(ws + WS_XT));
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
-    static const bool old_kernel = getenv("XMC_STEP_KERNEL") && !__builtin_strcmp(getenv("XMC_STEP_KERNEL"), "quad");
-    if (old_kernel) {
-      switch (round_mode) {
-        case XMC_ROUND_RTN: fp8_step_quad_kernel<ROUND_RTN><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
-        case XMC_ROUND_SR_PHILOX: fp8_step_quad_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
-        default: fp8_step_quad_kernel<ROUND_SR_FAST><<<qgrid, QNT, QLDS_BYTES, stream>>>(p); break;
-      }
-    } else {
-      switch (round_mode) {
-        case XMC_ROUND_RTN: fp8_step_role_kernel<ROUND_RTN><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
-        case XMC_ROUND_SR_PHILOX: fp8_step_role_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
-        default: fp8_step_role_kernel<ROUND_SR_FAST><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
-      }
+    switch (round_mode) {
+      case XMC_ROUND_RTN: fp8_step_role_kernel<ROUND_RTN><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+      case XMC_ROUND_SR_PHILOX: fp8_step_role_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+      default: fp8_step_role_kernel<ROUND_SR_FAST><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
-    if (old_kernel)
-      reduce_gx_quad_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
-                                                   (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
-    else
-      reduce_gx_role_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
-                                                   (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
+    reduce_gx_role_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
+                                                 (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
   }
   return launch_status();
 }
@@ -672,6 +659,8 @@ int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chun
 }
 
 size_t xmc_step_error_offset(void) { return WS_FLAGS + (size_t)QF_ERR * 4; }
+
+size_t xmc_step_sticky_error_offset(void) { return WS_FLAGS + (size_t)QF_STICKY * 4; }
 
 int xmc_step_workgroups(void) {
   DeviceInfo di = device_info();

@@ -35,6 +35,9 @@ constexpr int RC_RING = RQ + 1;             // own-column images: in use, RQ - 1
 #ifndef XMC_NB_B
 #define XMC_NB_B 3
 #endif
+#ifndef XMC_PD
+#define XMC_PD 3
+#endif
 constexpr int NB_B = XMC_NB_B;              // A^T blocks (16 label rows) of a tile the B wavefronts take; the A wavefronts take the rest
 constexpr int RR_RING = 3;                  // own-rows images: in use, landed, landing
 constexpr int RG_BUF = 2;                   // gathered G tiles: in use, landing
@@ -320,6 +323,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       // time; a key costs vector instructions only if it lies in this wavefront's block (label rows 16m.., batch rows
       // 32a..).  Up to seven keys behind the tile's last are read and ignored; the buffer behind the keys belongs to
       // the workspace.
+#ifndef XMC_X_NOPOS
       if (q.p1 > q.p0) {
         float sg[2][4];
 #pragma unroll
@@ -354,6 +358,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
           sb[blk][1] = bf16_pack2(sg[blk][2], sg[blk][3]);
         }
       }
+#endif
       if (q.rows_valid < TL) {   // rows past the end of the chunk contribute nothing
 #pragma unroll
         for (int blk = 0; blk < 2; blk++)
@@ -609,7 +614,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     // The operand of step k + 3 is requested in step k.  The vector work of the update of block o (12 weights per lane,
     // eight pieces) is spread over the steps behind the block's last, so that it issues between the matrix instructions.
     constexpr int NS = 16 + 4 * NB_B, NALT = 8 * NB_B;
-    bf16x8 op[NS + 3];
+    constexpr int PD = XMC_PD;   // operands are requested this many steps ahead
+    bf16x8 op[NS + PD];
     auto request = [&](int k) {
       if (k >= NS) return;
       if (k < NALT && (k & 1) == 0) {
@@ -620,7 +626,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       }
     };
     const int abort_word = *(const lds_int*)(lds + abort_base + ((i + 1) & 1) * 4);
-    request(0); request(1); request(2);
+#pragma unroll
+    for (int k = 0; k < PD; k++) request(k);
     intx2 wraw[2][3];
 #pragma unroll
     for (int ks2 = 0; ks2 < 2; ks2++)
@@ -642,9 +649,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       if ((k & 7) == 1 && k < 24) so_v = so_read((i + 1) & 1, k >> 3);
       if ((k & 7) == 5 && k < 24) so_store(q_p, k >> 3, so_v);
 #ifndef XMC_X_NOBLDS
-      request(k + 3);
+      request(k + PD);
 #else
-      if (k + 3 < NS) op[k + 3] = op[k & 1];
+      if (k + PD < NS) op[k + PD] = op[k & 1];
 #endif
       // vector pieces of this step
       if (k == 0) {
@@ -681,7 +688,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 #pragma unroll
         for (int nn = 0; nn < 3; nn++) acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op[k], wb[ks2][nn], acc2[mb][nn], 0, 0, 0);
       }
+#ifndef XMC_X_NOBFENCE
       QFENCE();
+#endif
     }
     if (NB_B == 4) {
 #pragma unroll
@@ -713,8 +722,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
                                                              unsigned short* gx_bf16, int batch, int* flags) {
   // placement check: the members of a quad exchanged G through the L2 of one XCD, which holds only if all four ran there
-  if (blockIdx.x == 0 && (int)threadIdx.x < (nwg >> 2) && quad_xcc_mismatch(flags + QF_XCC, (int)threadIdx.x))
-    __hip_atomic_fetch_or(flags + QF_ERR, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (blockIdx.x == 0) {
+    if ((int)threadIdx.x < (nwg >> 2) && quad_xcc_mismatch(flags + QF_XCC, (int)threadIdx.x))
+      __hip_atomic_fetch_or(flags + QF_ERR, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    // the error word of this step joins the sticky word, which no kernel clears: a caller that looks at it only now and
+    // then still learns of every failed step
+    if (threadIdx.x == 0) {
+      const int e = __hip_atomic_load(flags + QF_ERR, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (e != 0) __hip_atomic_fetch_or(flags + QF_STICKY, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
   const int blk = blockIdx.x >> 3, m = (blockIdx.x >> 1) & 3;   // blk = mb*3+nn
   const int t = (blockIdx.x & 1) * 128 + threadIdx.x, s = t >> 6, lane = t & 63, l16 = lane & 15, kg = lane >> 4;
   // the workgroups of member m, in a fixed order; eight loads in flight at a time

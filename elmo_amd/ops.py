@@ -33,7 +33,11 @@ def workspace_bytes(num_chunks, rows_per_chunk):
 
 
 def alloc_workspace(num_chunks, rows_per_chunk, device):
-    return torch.empty(workspace_bytes(num_chunks, rows_per_chunk), dtype=torch.uint8, device=device)
+    ws = torch.empty(workspace_bytes(num_chunks, rows_per_chunk), dtype=torch.uint8, device=device)
+    # the sticky error word is only ever OR-ed into by the kernels: it starts at zero
+    off = step_sticky_error_offset()
+    ws[off:off + 4].zero_()
+    return ws
 
 
 def fp8_step(chunks, x, labels, lr, seeds=None, round_mode="rtn", scale_w=1.0, scale_x=1.0, workspace=None,
@@ -263,6 +267,11 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
 def step_error_offset():
     """Byte offset of the fused step's error word (int32) inside its workspace."""
     return int(_lib.load().xmc_step_error_offset())
+
+
+def step_sticky_error_offset():
+    """Byte offset of the sticky error word (int32): the error words of all fused steps since it was last zeroed."""
+    return int(_lib.load().xmc_step_sticky_error_offset())
 
 
 def step_error_word(workspace, num_chunks, rows_per_chunk):

@@ -81,12 +81,16 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
         self._tiled_workspace = None
         self._fused_ran = False      # the error word in the workspace is defined once a fused step has run
-        # After every fused step the error word is copied to pinned host memory on the step's stream, without waiting;
-        # the next step looks at copies that have arrived (see _check_previous_steps).
-        off = ops.step_error_offset()
+        # After every fused step the workspace's sticky error word (the error words of all steps since it was last
+        # zeroed, OR-ed together by the kernels) is copied to pinned host memory on the step's stream, without waiting;
+        # later calls look at the copies that have arrived (see _check_previous_steps).  A ring of slots, so that a copy
+        # still in flight is never overwritten by the next one.
+        off = ops.step_sticky_error_offset()
         self._err_dev = self._workspace[off:off + 4].view(torch.int32)
-        self._err_host = torch.zeros(1, dtype=torch.int32).pin_memory()
-        self._err_event = None
+        self._err_slots = 4
+        self._err_host = torch.zeros(self._err_slots, dtype=torch.int32).pin_memory()
+        self._err_events = [None] * self._err_slots
+        self._err_next = 0
         # batches of more than 128 rows (up to 512) also run on the three-kernel path, with the true-FP8 arithmetic
         self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
@@ -180,25 +184,46 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
                                            scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
             self._fused_ran = True
-            # the step's error word follows it on the stream into pinned host memory; nobody waits for it here
-            self._err_host.copy_(self._err_dev, non_blocking=True)
-            self._err_event = torch.cuda.Event()
-            self._err_event.record()
+            # the sticky error word follows the step on the stream into pinned host memory; nobody waits for it here
+            slot = self._err_next
+            if self._err_events[slot] is not None:
+                self._err_events[slot].synchronize()      # that copy was enqueued four steps ago
+                self._raise_on_error(int(self._err_host[slot]))
+            self._err_host[slot:slot + 1].copy_(self._err_dev, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            self._err_events[slot] = ev
+            self._err_next = (slot + 1) % self._err_slots
         self.iteration += 1
         return loss
 
+    def _raise_on_error(self, word):
+        if word != 0:
+            self._err_dev.zero_()                 # on the stream, behind every step enqueued so far
+            self._err_host.zero_()
+            self._err_events = [None] * self._err_slots
+            raise RuntimeError(
+                f"a fused classifier step failed (error word {word}): "
+                + ("a workgroup gave up waiting for its partners (another stream kept the device busy?); " if word & 1 else "")
+                + ("the workgroups of a quad were not placed on one XCD; " if word & 2 else "")
+                + "the weights and grad_input of that step are incomplete")
+
     def _check_previous_steps(self):
-        """Raises if a fused step whose error word has reached the host reported a failure (never waits: a word that is
-        still on its way is looked at by a later call)."""
-        if self._err_event is not None and self._err_event.query():
-            word = int(self._err_host[0])
-            if word != 0:
-                self._err_host[0] = 0
-                raise RuntimeError(
-                    f"fused classifier step failed (error word {word}): "
-                    + ("a workgroup gave up waiting for its partners (another stream kept the device busy?); " if word & 1 else "")
-                    + ("the workgroups of a quad were not placed on one XCD; " if word & 2 else "")
-                    + "the weights and grad_input of that step are incomplete")
+        """Raises if a fused step reported a failure and a copy of the sticky error word taken behind it has reached the
+        host.  Never waits: a copy that is still on its way is looked at by a later call.  The word is sticky, so a
+        failure is not lost when later, clean steps have run in between."""
+        for slot in range(self._err_slots):
+            ev = self._err_events[slot]
+            if ev is not None and ev.query():
+                self._err_events[slot] = None
+                self._raise_on_error(int(self._err_host[slot]))
+
+    def check_steps(self):
+        """Waits for the steps enqueued so far and raises if any of them failed (the end of a run, a checkpoint).  Not
+        part of the reference's interface."""
+        if self._fused_ran:
+            torch.cuda.current_stream().synchronize()
+            self._raise_on_error(int(self._err_dev.item()))
 
     def last_step_error(self):
         """Error word of the last fused step (0 = fine; non-zero = a workgroup gave up waiting for its partners, e.g.

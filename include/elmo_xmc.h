@@ -202,9 +202,15 @@ int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
  * Synchronises the stream: meant for tests, debugging and a check where the training loop synchronises anyway. */
 int xmc_step_error_word(const void* workspace, int num_chunks, int rows_per_chunk, void* stream);
 
-/* Byte offset of that error word (one int32) inside the workspace, for callers that want to copy it to pinned host
- * memory asynchronously after every step instead of synchronising (the Python module does). */
+/* Byte offset of that error word (one int32) inside the workspace. */
 size_t xmc_step_error_offset(void);
+
+/* Byte offset of the sticky error word (one int32) inside the workspace (no counterpart in the reference): the last
+ * kernel of every fused step ORs the step's error word into it, and no kernel ever clears it.  It is for callers that
+ * do not want to synchronise after every step: zero the word once after allocating the workspace, copy it to pinned
+ * host memory behind any step (or every few steps) without waiting, and look at a copy whenever one has arrived - a
+ * failure of any step since the word was last zeroed is still in it.  Zero it again after handling a failure. */
+size_t xmc_step_sticky_error_offset(void);
 
 /* Diagnostics of the placement assumption of the fused kernel (no counterpart in the reference).  The kernel builds
  * quads out of workgroups g with equal g % 8 and expects them on one XCD; every workgroup records the XCC id it really
