@@ -23,21 +23,21 @@ def load():
         raise XmcError(
             f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
             "(hipcc --offload-arch=gfx950); there is no CPU fallback for the classifier step")
-    lib = ctypes.CDLL(LIB_PATH)
-    # a library that predates an edit of the sources would run the old kernels: it reports the digest of the sources it
-    # was compiled from; on a mismatch it is rebuilt once, and if that is not possible the load fails
-    lib.xmc_source_hash.restype = ctypes.c_char_p
+    # A library that predates an edit of the sources would run the old kernels.  build() leaves the digest of the sources
+    # beside the library; it is compared BEFORE the library is loaded, because a loaded library cannot be replaced within
+    # the process (loading the same path again returns the mapping that is already there).  On a mismatch the library
+    # is rebuilt under a temporary name and moved into place, then loaded.
     from . import build as _build
-    if LIB_PATH == _build.OUT and lib.xmc_source_hash().decode() != _build.source_hash():
-        del lib
+    if LIB_PATH == _build.OUT and _build.built_hash() != _build.source_hash():
         try:
             _build.build()
         except Exception as e:
             raise XmcError(f"{LIB_PATH} was built from other sources than those in the tree and could not be rebuilt: {e}")
-        lib = ctypes.CDLL(LIB_PATH)
-        lib.xmc_source_hash.restype = ctypes.c_char_p
-        if lib.xmc_source_hash().decode() != _build.source_hash():
-            raise XmcError(f"{LIB_PATH} does not match the sources in the tree even after a rebuild")
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.xmc_source_hash.restype = ctypes.c_char_p
+    if LIB_PATH == _build.OUT and lib.xmc_source_hash().decode() != _build.source_hash():
+        raise XmcError(f"{LIB_PATH} reports other sources than those in the tree: rebuild it "
+                       "(python -c 'import __graft_entry__ as g; g.build()') and start the process again")
     vp, i32, f32, sz, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_longlong
     lib.xmc_version.restype = i32
     lib.xmc_source_hash.restype = ctypes.c_char_p

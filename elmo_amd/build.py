@@ -28,14 +28,34 @@ def source_hash():
     return h.hexdigest()[:16]
 
 
+HASH_FILE = OUT + ".hash"
+
+
+def built_hash():
+    """Digest of the sources the library in the tree was built from (written by build()), or None."""
+    try:
+        with open(HASH_FILE) as f:
+            return f.read().strip()
+    except OSError:
+        return None
+
+
 def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + [f'-DXMC_SOURCE_HASH="{source_hash()}"', SRC, "-o", OUT]
+    digest = source_hash()
+    tmp = OUT + ".tmp%d" % os.getpid()
+    cmd = [hipcc] + HIPCC_FLAGS + [f'-DXMC_SOURCE_HASH="{digest}"', SRC, "-o", tmp]
     if verbose:
         cmd.append("-Rpass-analysis=kernel-resource-usage")
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
         raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+    # moved into place in one step: a process that has the previous library mapped keeps its (unlinked) file
+    os.replace(tmp, OUT)
+    with open(HASH_FILE, "w") as f:
+        f.write(digest + "\n")
     return res.stderr if verbose else OUT
 
 

@@ -8,6 +8,7 @@
 #include "xmc_topk.hip"
 #include "xmc_dropout.hip"
 #include <stdlib.h>
+#include <mutex>
 
 using namespace xmc;
 
@@ -24,46 +25,53 @@ namespace {
 
 struct DeviceInfo { int ok; int cus; unsigned char* scratch_ptr; };
 
+// Filled once per device, by the first call on it; std::call_once makes concurrent first calls of several host threads
+// wait for the one that fills the slot, and publishes the finished slot to all of them.
+DeviceInfo g_device_info[64];
+std::once_flag g_device_once[64];
+
+void fill_device_info(int dev) {
+  DeviceInfo di = {-1, 0, nullptr};
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) { g_device_info[dev] = di; return; }
+  di.cus = prop.multiProcessorCount;
+  di.ok = (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : -1;
+  // this device's copy of the static scratch array (device `dev` is current here); stays null if the lookup fails
+  void* sp = nullptr;
+  di.scratch_ptr = (di.ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess) ? (unsigned char*)sp : nullptr;
+  // opt in to the full 160 KiB of LDS once per device
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
+  (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
+  (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
+  (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
+  (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 2>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+  (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
+  (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
+  (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
+  // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
+#define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
+  XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_FAST, false);
+  XMC_UPD_ATTR(W_E4M3, ROUND_RTN, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, false);
+  XMC_UPD_ATTR(W_E4M3, ROUND_RTN, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, true);
+#undef XMC_UPD_ATTR
+  g_device_info[dev] = di;
+}
+
 DeviceInfo device_info() {
-  static DeviceInfo cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return DeviceInfo{-1, 0, nullptr};
-  if (cached[dev].ok == 0) {
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DeviceInfo{-1, 0, nullptr};
-    cached[dev].cus = prop.multiProcessorCount;
-    cached[dev].ok = (__builtin_strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : -1;
-    // this device's copy of the static scratch array (device `dev` is current here); stays null if the lookup fails
-    void* sp = nullptr;
-    cached[dev].scratch_ptr = (cached[dev].ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess)
-                                  ? (unsigned char*)sp : nullptr;
-    // opt in to the full 160 KiB of LDS once per device
-    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-    (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
-    (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
-    (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
-    (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
-    (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
-    (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 2>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
-    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
-    (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
-    // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
-#define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
-    XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_FAST, false);
-    XMC_UPD_ATTR(W_E4M3, ROUND_RTN, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, false);
-    XMC_UPD_ATTR(W_E4M3, ROUND_RTN, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, true);
-#undef XMC_UPD_ATTR
-  }
-  return cached[dev];
+  std::call_once(g_device_once[dev], fill_device_info, dev);
+  return g_device_info[dev];
 }
 
 // optional event pair recorded around the next launch of the fused step kernel by the calling thread (benchmarking aid)

@@ -570,6 +570,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     typedef __attribute__((address_space(1))) intx4 gi4;
     unsigned char* dst = so_row[jj] < qp.rows_valid ? qp.base + so_mem[jj] : bl.dummy;
 #ifndef XMC_X_NOSTORE
+    // plain stores on purpose: non-temporal ones keep the exchanged G tiles and the tiles between their two fetches in
+    // the XCD's L2 (reads from memory drop from 1.34 to 1.05 times the weights) but cost 5 % of the kernel's time
     *(gi4*)(unsigned long long)dst = ov;
 #else
     if (ov.x == 0x12345) *(gi4*)(unsigned long long)dst = ov;
