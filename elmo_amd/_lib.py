@@ -48,6 +48,9 @@ def load():
     lib.xmc_fp8_step.restype = i32
     lib.xmc_fp8_step.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, vp, i32, f32,
                                  ctypes.POINTER(ctypes.c_uint32), i32, f32, f32, vp, vp, vp, sz, vp]
+    lib.xmc_fp8_step_ex.restype = i32
+    lib.xmc_fp8_step_ex.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, vp, i32, f32,
+                                    ctypes.POINTER(ctypes.c_uint32), i32, f32, f32, f32, f32, ctypes.c_ulonglong, vp, vp, vp, sz, vp]
     lib.xmc_fp8_forward.restype = i32
     lib.xmc_fp8_forward.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp, sz, vp]
     lib.xmc_fp8_forward_static.restype = i32
@@ -59,6 +62,10 @@ def load():
     lib.xmc_tiled_step.restype = i32
     lib.xmc_tiled_step.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32, vp, i32, i32, vp, i32, f32,
                                    ctypes.POINTER(ctypes.c_uint32), i32, i32, i32, vp, i32, i32, vp, vp, vp, vp, sz, vp]
+    lib.xmc_tiled_step_ex.restype = i32
+    lib.xmc_tiled_step_ex.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32, vp, i32, i32, vp, i32, f32,
+                                      ctypes.POINTER(ctypes.c_uint32), i32, i32, i32, vp, i32, i32, f32, f32, ctypes.c_ulonglong,
+                                      vp, vp, vp, vp, sz, vp]
     lib.xmc_topk_scratch_bytes.restype = sz
     lib.xmc_topk_scratch_bytes.argtypes = [i32]
     lib.xmc_fp8_forward_topk.restype = i32

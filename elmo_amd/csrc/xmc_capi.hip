@@ -40,9 +40,12 @@ void fill_device_info(int dev) {
   void* sp = nullptr;
   di.scratch_ptr = (di.ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess) ? (unsigned char*)sp : nullptr;
   // opt in to the full 160 KiB of LDS once per device
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
   (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
@@ -180,6 +183,14 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
                  int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
                  float scale_w, float scale_x, void* grad_x_bf16, float* grad_x_f32, void* workspace,
                  size_t workspace_bytes, void* stream_) {
+  return xmc_fp8_step_ex(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, labels_coo, nnz, lr, seeds, round_mode,
+                         scale_w, scale_x, 0.0f, 0.0f, 0ull, grad_x_bf16, grad_x_f32, workspace, workspace_bytes, stream_);
+}
+
+int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                    int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                    float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
+                    void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream_) {
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
   if (!grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
@@ -188,10 +199,12 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   if (round_mode < XMC_ROUND_RTN || round_mode > XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
   if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
+  if (!(weight_decay >= 0.f) || !(dropout_p >= 0.f) || !(dropout_p < 1.f)) return XMC_ERR_SHAPE;
   DeviceInfo di = device_info();
   if (di.ok != 1 || di.cus < 16) return XMC_ERR_DEVICE;
   hipStream_t stream = (hipStream_t)stream_;
   unsigned char* ws = (unsigned char*)workspace;
+  const DropoutParams dp = {dropout_p, 1.0f - dropout_p, (unsigned)(dropout_seed & 0xFFFFFFFFull), (unsigned)(dropout_seed >> 32)};
 
   const int grid = di.cus < MAX_WG ? di.cus : MAX_WG;   // one workgroup per compute unit
   const int tiles_per_chunk = (rows_per_chunk + TL - 1) / TL;
@@ -220,6 +233,7 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     p.flags = (int*)(ws + WS_FLAGS);
     p.zscale = scale_w * scale_x;
     p.lr_eff = lr / scale_w;
+    p.wd_eff = weight_decay * scale_w;   // T = c - (lr / s) (A + wd s c) for codes c = W / s
     p.batch = batch;
     int qgrid = grid / 32 * 32;   // whole quads on every XCD
 #ifdef XMC_DEV_GRID
@@ -233,17 +247,23 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
     quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, (size_t)(n_pad + 257) * 4, stream>>>(
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
-        (unsigned short*)(ws + WS_XT));
+        (unsigned short*)(ws + WS_XT), dp);
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
+#define XMC_LAUNCH_STEP(RMODE)                                                                             \
+  do {                                                                                                     \
+    if (weight_decay != 0.f) fp8_step_role_kernel<RMODE, true><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);     \
+    else fp8_step_role_kernel<RMODE, false><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);                        \
+  } while (0)
     switch (round_mode) {
-      case XMC_ROUND_RTN: fp8_step_role_kernel<ROUND_RTN><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
-      case XMC_ROUND_SR_PHILOX: fp8_step_role_kernel<ROUND_SR_PHILOX><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
-      default: fp8_step_role_kernel<ROUND_SR_FAST><<<qgrid, QNT, RLDS_BYTES, stream>>>(p); break;
+      case XMC_ROUND_RTN: XMC_LAUNCH_STEP(ROUND_RTN); break;
+      case XMC_ROUND_SR_PHILOX: XMC_LAUNCH_STEP(ROUND_SR_PHILOX); break;
+      default: XMC_LAUNCH_STEP(ROUND_SR_FAST); break;
     }
+#undef XMC_LAUNCH_STEP
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
     reduce_gx_role_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
-                                                 (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS));
+                                                 (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS), dp);
   }
   return launch_status();
 }
@@ -481,6 +501,16 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
                    const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
                    int num_head, void* grad_x_bf16, float* grad_x_f32, float* loss_out, void* workspace,
                    size_t workspace_bytes, void* stream_) {
+  return xmc_tiled_step_ex(chunk_ptrs, num_chunks, rows_per_chunk, rows_last_chunk, weight_type, x_bf16, batch, features, labels_coo,
+                           nnz, lr, seeds, round_mode, quantize_x, saturate, kahan, kahan_type, num_head, 0.0f, 0.0f, 0ull,
+                           grad_x_bf16, grad_x_f32, loss_out, workspace, workspace_bytes, stream_);
+}
+
+int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                      const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
+                      const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                      int num_head, float weight_decay, float dropout_p, unsigned long long dropout_seed, void* grad_x_bf16,
+                      float* grad_x_f32, float* loss_out, void* workspace, size_t workspace_bytes, void* stream_) {
   if (!chunk_ptrs || !x_bf16 || !workspace || !grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
   if (kahan_type < 0 || kahan_type > 2 || (kahan_type != 0 && (weight_type != W_E4M3 || !kahan))) return XMC_ERR_MODE;
   if (kahan_type != 0 && (num_head < 0 || num_head > rows_per_chunk || !aligned16(kahan))) return XMC_ERR_SHAPE;
@@ -492,6 +522,10 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   if (weight_type != W_E4M3 && weight_type != W_BF16) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX && round_mode != XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
+  if (!(weight_decay >= 0.f) || !(dropout_p >= 0.f) || !(dropout_p < 1.f)) return XMC_ERR_SHAPE;
+  if (kahan_type != 0 && (weight_decay != 0.f || dropout_p != 0.f)) return XMC_ERR_MODE;   // the head-Kahan layer has neither
+  const DropoutParams dp = {dropout_p, 1.0f - dropout_p, (unsigned)(dropout_seed & 0xFFFFFFFFull), (unsigned)(dropout_seed >> 32)};
+  const float wd = weight_decay;
   for (int c = 0; c < num_chunks; c++) {
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
@@ -544,7 +578,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
   const bool split_update = weight_type == W_E4M3 && halves == 2 && kahan_type == 0;
   tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x,
                                                                         fp8_logits ? 1 : 0, split_update ? 1 : 0, xb, xT, gx_total,
-                                                                        loss_part, loss_out ? 2 * num_tiles : 0);
+                                                                        loss_part, loss_out ? 2 * num_tiles : 0, dp);
   for (int c = 0; c < num_chunks; c += group) {
     void* w = chunk_ptrs[c];
     const int nch = c + group <= num_chunks ? group : num_chunks - c;                       // chunks of this launch
@@ -607,7 +641,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
     const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) + (12 / tup_csteps(halves)) * ((ugroups + 7) / 8 * 8);
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
   tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV), stream>>>(                           \
-      w, rows, tiles, glb, g_half, xT, lr, sd, cs, saturate, kahan, kahan_type, nh, label0, partial, part_half, nch, spc, range, rp,  \
+      w, rows, tiles, glb, g_half, xT, lr, wd, sd, cs, saturate, kahan, kahan_type, nh, label0, partial, part_half, nch, spc, range, rp,  \
       weight_type == W_BF16 ? 1 : 0, gx_total)
 #define XMC_LAUNCH_UPDATE_H(WTYPE, RMODE, KH)                                                                                  \
   do {                                                                                                                         \
@@ -621,7 +655,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
       streams = streams < 128 ? streams : 128;           // two workgroups per compute unit, four per stream
       const int grid2 = TRED_WAVES * 2 / 4 + 4 * streams;
 #define XMC_LAUNCH_UPDATE2(RMODE)                                                                                              \
-  tiled_update2_kernel<RMODE><<<grid2, 256, 2 * TU2_GBUF, stream>>>(w, rows, tiles, glb, g_half, (const bf16x8*)xT, lr, sd, cs, saturate, \
+  tiled_update2_kernel<RMODE><<<grid2, 256, 2 * TU2_GBUF, stream>>>(w, rows, tiles, glb, g_half, (const bf16x8*)xT, lr, wd, sd, cs, saturate, \
                                                                     label0, partial, part_half, nch, spc, range, rp, gx_total)
       if (round_mode == XMC_ROUND_RTN) XMC_LAUNCH_UPDATE2(ROUND_RTN);
       else if (round_mode == XMC_ROUND_SR_FAST) XMC_LAUNCH_UPDATE2(ROUND_SR_FAST);
@@ -643,7 +677,7 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
 #undef XMC_LAUNCH_UPDATE_H
 #undef XMC_LAUNCH_UPDATE_K
   }
-  tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32);
+  tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32, dp);
   if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, 2 * num_tiles, loss_out);
   return launch_status();
 }

@@ -106,6 +106,27 @@ __device__ __forceinline__ unsigned fast_word(unsigned h, int i) {
   return h * k[i];
 }
 
+// Dropout of the embedding inside the step (training.xmc dropout fused into the preparation of X; the reference keeps a
+// prototype of this in src/triton_kernels/tma_gemm.py:7-13): element (b, k) is kept when rand(seed, b * D + k) > p, rand
+// being Triton's tl.rand (first Philox-4x32-10 word of counter (offset, 0, 0, 0), key = seed, as a uniform fp32).
+struct DropoutParams { float p; float keep_scale; unsigned seed_lo, seed_hi; };   // p == 0: no dropout
+
+__device__ __forceinline__ bool dropout_keep(unsigned off, const DropoutParams& dp) {
+  int r = (int)philox_word0(off, dp.seed_lo, dp.seed_hi);
+  r = r < 0 ? -r - 1 : r;
+  return (float)r * 4.6566127342e-10f > dp.p;
+}
+// the dropped-out embedding in the layer's type: bf16(keep ? x / (1 - p) : 0)
+__device__ __forceinline__ unsigned short dropout_bf16(unsigned short raw, unsigned off, const DropoutParams& dp) {
+  if (dp.p == 0.f) return raw;
+  return dropout_keep(off, dp) ? bf16_bits(bf16_from_bits(raw) / dp.keep_scale) : (unsigned short)0;
+}
+// gradient with respect to the embedding in front of the dropout
+__device__ __forceinline__ float dropout_backward(float g, unsigned off, const DropoutParams& dp) {
+  if (dp.p == 0.f) return g;
+  return dropout_keep(off, dp) ? g / dp.keep_scale : 0.f;
+}
+
 enum RoundMode { ROUND_RTN = 0, ROUND_SR_PHILOX = 1, ROUND_SR_FAST = 2 };
 
 // Round four updated weights (fp32) of one row, columns col..col+3, to e4m3 codes packed in a dword.

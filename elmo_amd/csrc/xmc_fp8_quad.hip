@@ -47,6 +47,7 @@ struct QuadParams {
   int* flags;                         // [nquads][16] tiles-published counters; [QF_XCC + g] XCC ids; [QF_ERR] error word
   float zscale;                       // scale_w * scale_x applied to the logits accumulator
   float lr_eff;                       // lr / scale_w
+  float wd_eff;                       // weight decay x scale_w (applied to the codes)
   int batch;
 };
 
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
 }
 
 __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
-                                                   unsigned short* xt);
+                                                   unsigned short* xt, const DropoutParams& dp);
 
 // Second launch: blocks below desc_blocks write, for every tile,
 //   desc[t] = {base pointer, valid rows, seed | first key, one past the last key, row in chunk, first label}
@@ -191,9 +192,9 @@ __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* 
 // and the remaining blocks build the operand images of X.
 __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p, int n_pad, int* tile_ptr, uint4* desc, int desc_blocks,
                                                              const unsigned short* x, float inv_scale_x, unsigned char* xq,
-                                                             unsigned short* xt) {
+                                                             unsigned short* xt, const DropoutParams dp) {
   if ((int)blockIdx.x >= desc_blocks) {
-    prep_x_quad_thread(((int)blockIdx.x - desc_blocks) * 256 + (int)threadIdx.x, x, p.batch, inv_scale_x, xq, xt);
+    prep_x_quad_thread(((int)blockIdx.x - desc_blocks) * 256 + (int)threadIdx.x, x, p.batch, inv_scale_x, xq, xt, dp);
     return;
   }
   // the sorted keys go to LDS first (n_pad * 4 bytes, then 257 search results): a binary search in global memory
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
 //   xt: bf16 X^T in v_mfma 16x16x32 A-operand order: [((col/48)*3 + cg)*4 + ks][lane][8 bf16], lane = r + 16*kg,
 //       element j = X[32ks + 8kg + j][col] with col = 48*(col/48) + 12*(r/4) + 4*cg + r%4
 __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* x, int batch, float inv_scale_x, unsigned char* xq,
-                                                   unsigned short* xt) {
+                                                   unsigned short* xt, const DropoutParams& dp) {
   // one thread per (b, group of 4 features)
   if (i >= BP * (D / 4)) return;
   int b = i / (D / 4), k = (i - b * (D / 4)) * 4;
@@ -256,7 +257,10 @@ __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* 
   unsigned short raw[4] = {0, 0, 0, 0};
   if (b < batch) {
 #pragma unroll
-    for (int q = 0; q < 4; q++) { raw[q] = x[(size_t)b * D + k + q]; v[q] = bf16_from_bits(raw[q]) * inv_scale_x; }
+    for (int q = 0; q < 4; q++) {   // with dropout, both images are those of the dropped-out embedding
+      raw[q] = dropout_bf16(x[(size_t)b * D + k + q], (unsigned)(b * D + k + q), dp);
+      v[q] = bf16_from_bits(raw[q]) * inv_scale_x;
+    }
   }
   int packed = 0;
   packed = __builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v[0]), clamp448(v[1]), packed, false);

@@ -86,10 +86,10 @@ struct RBlockLane {
 // piece c (0..7) of the update of A^T block nb (12 weights per lane): pieces 0-2 decode the old weights and form
 // T = W - lr A, 3-5 make the random words' hashes, 6-7 round, 7 stores.  Split so that the vector instructions can be
 // issued between matrix instructions.  With MODE.FP16_OVFL set the fp8 converters saturate, so nothing is clamped here.
-template <int MODE>
+template <int MODE, bool WD>
 __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab)[3], const unsigned (&wq)[3], float (&t)[3][4],
                                                unsigned (&hs)[3], unsigned (&outw)[3], const RBlockLane& bl, const QTile& q,
-                                               unsigned hash_tile, float lr_eff, int l16, qlds_u8* lds, unsigned oimg) {
+                                               unsigned hash_tile, float lr_eff, float wd_eff, int l16, qlds_u8* lds, unsigned oimg) {
 #ifdef XMC_X_NOUPDATE
   if (c == 7 && ab[0][0] + ab[1][1] + ab[2][2] == 1.2345f) *(volatile unsigned*)bl.dummy = wq[0] + wq[1] + wq[2];
   return;
@@ -98,8 +98,15 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
     const int cg = c;
     const unsigned wv = wq[cg];
     floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, true);
-    t[cg][0] = __builtin_fmaf(-lr_eff, ab[cg][0], w01.x); t[cg][1] = __builtin_fmaf(-lr_eff, ab[cg][1], w01.y);
-    t[cg][2] = __builtin_fmaf(-lr_eff, ab[cg][2], w23.x); t[cg][3] = __builtin_fmaf(-lr_eff, ab[cg][3], w23.y);
+    if (WD) {   // T = W - lr (A + wd W): the decayed gradient first, in fp32
+      t[cg][0] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w01.x, ab[cg][0]), w01.x);
+      t[cg][1] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w01.y, ab[cg][1]), w01.y);
+      t[cg][2] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w23.x, ab[cg][2]), w23.x);
+      t[cg][3] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w23.y, ab[cg][3]), w23.y);
+    } else {
+      t[cg][0] = __builtin_fmaf(-lr_eff, ab[cg][0], w01.x); t[cg][1] = __builtin_fmaf(-lr_eff, ab[cg][1], w01.y);
+      t[cg][2] = __builtin_fmaf(-lr_eff, ab[cg][2], w23.x); t[cg][3] = __builtin_fmaf(-lr_eff, ab[cg][3], w23.y);
+    }
   } else if (c < 6) {
     const int cg = c - 3;
     if (MODE == ROUND_SR_FAST) {
@@ -138,7 +145,7 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
   }
 }
 
-template <int MODE>
+template <int MODE, bool WD>
 __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   qlds_u8* lds = (qlds_u8*)lds_raw;
@@ -502,7 +509,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
             constexpr int every = 2 * (4 - NB_B);
             const int pc = (nb - NB_B) * 8 + c;
             if (pc % every == 0) rows_piece(rslot, qr, pc / every);
-            r_update_piece<MODE>(c, nb, aa[nb - NB_B], wq[nb - NB_B], t, hs, outw, bl, qb, hash_tile, p.lr_eff, l16, lds, oimg);
+            r_update_piece<MODE, WD>(c, nb, aa[nb - NB_B], wq[nb - NB_B], t, hs, outw, bl, qb, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
           }
         if (NB_B == 4) rows_pieces(rslot, qr);
       }
@@ -671,13 +678,13 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       }
       if (k >= 8 && k < NALT) {
         const int o = (k >> 3) - 1;
-        r_update_piece<MODE>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, l16, lds, oimg);
+        r_update_piece<MODE, WD>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
       } else if (k >= NALT && NB_B > 0) {
         constexpr int per = NB_B == 4 ? 8 : 8 / (16 - 4 * NB_B);   // pieces per trailing step
         const int o = NB_B - 1;
 #pragma unroll
         for (int c = (k - NALT) * per; c < (k - NALT + 1) * per && c < 8; c++)
-          r_update_piece<MODE>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, l16, lds, oimg);
+          r_update_piece<MODE, WD>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
       }
       if (k < NALT && (k & 1) == 0) {
         const int o = k >> 3, ks = (k & 7) >> 1;
@@ -696,7 +703,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     }
     if (NB_B == 4) {
 #pragma unroll
-      for (int c = 0; c < 8; c++) r_update_piece<MODE>(c, 3, aa[1], wq[1], t, hs, outw, bl, q, hash_tile, p.lr_eff, l16, lds, oimg);
+      for (int c = 0; c < 8; c++) r_update_piece<MODE, WD>(c, 3, aa[1], wq[1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
     }
     q_p = q;
     q_n = q_desc_full(cdesc, tile_at(i + 1));
@@ -722,7 +729,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 // grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768].  192 workgroups of 128
 // threads: workgroup (block, m, part) covers lanes 128 part.. of the 256 B-wavefront lanes of a step workgroup.
 __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
-                                                             unsigned short* gx_bf16, int batch, int* flags) {
+                                                             unsigned short* gx_bf16, int batch, int* flags, const DropoutParams dp) {
   // placement check: the members of a quad exchanged G through the L2 of one XCD, which holds only if all four ran there
   if (blockIdx.x == 0) {
     if ((int)threadIdx.x < (nwg >> 2) && quad_xcc_mismatch(flags + QF_XCC, (int)threadIdx.x))
@@ -753,7 +760,7 @@ __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* part
   for (int i = 0; i < 4; i++) {
     const int b = 16 * mb + 4 * kg + i;
     if (b < batch) {
-      const float val = sum[i] * scale;
+      const float val = dropout_backward(sum[i] * scale, (unsigned)(b * D + col), dp);
       if (gx_f32) gx_f32[(size_t)b * D + col] = val;
       if (gx_bf16) gx_bf16[(size_t)b * D + col] = bf16_bits(val);
     }

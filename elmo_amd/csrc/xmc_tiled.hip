@@ -82,13 +82,14 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 // xt_split (two halves only): xT in the order of tiled_update2_kernel instead, [feature quarter][wavefront][block cg][K step
 // of 32 batch rows, 8 over both halves][lane][8], row 4kq + e of block cg being feature 12kq + 4cg + e of the wavefront's 48.
 __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, int fp8_image, int xt_split,
-                                    unsigned short* xb, unsigned short* xT, float* gx_total, float* loss_part, int n_loss) {
+                                    unsigned short* xb, unsigned short* xT, float* gx_total, float* loss_part, int n_loss,
+                                    const DropoutParams dp) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= halves * BP * D) return;
   gx_total[i] = 0.f;
   for (int j = i; j < n_loss; j += halves * BP * D) loss_part[j] = 0.f;
   int b = i / D, k = i - b * D;
-  unsigned short v = b < batch ? x[(size_t)b * D + k] : (unsigned short)0;
+  unsigned short v = b < batch ? dropout_bf16(x[(size_t)b * D + k], (unsigned)i, dp) : (unsigned short)0;
   unsigned short vq = v;
   int code = 0;
   if (quantize) {
@@ -616,10 +617,10 @@ __device__ __forceinline__ void tiled_reduce_wave(int widx, int lane, const floa
   }
 }
 
-__global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned short* gx_bf16, float* gx_f32) {
+__global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned short* gx_bf16, float* gx_f32, const DropoutParams dp) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= batch * D) return;
-  const float v = gx_total[i];
+  const float v = dropout_backward(gx_total[i], (unsigned)i, dp);
   if (gx_f32) gx_f32[i] = v;
   gx_bf16[i] = bf16_bits(v);
 }
@@ -638,7 +639,7 @@ __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned
 // Four consecutive features of one row: old weights (bf16: two dwords, e4m3: one) and compensation terms in, new ones out.
 template <int WT, int MODE>
 __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const unsigned* kraw, bool head, int kahan_type, float lr,
-                                          unsigned off0, unsigned fidx, unsigned seed, int saturate, unsigned* wout, unsigned* kout) {
+                                          float wd, unsigned off0, unsigned fidx, unsigned seed, int saturate, unsigned* wout, unsigned* kout) {
   float wv4[4];
   if (WT == W_BF16) {
     wv4[0] = bf16_from_bits((unsigned short)(wraw[0] & 0xffffu)); wv4[1] = bf16_from_bits((unsigned short)(wraw[0] >> 16));
@@ -660,7 +661,9 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
   float t[4];
 #pragma unroll
   for (int e = 0; e < 4; e++) {
-    const float g = WT == W_BF16 ? bf16_rt(a[e]) : a[e];
+    // the gradient plus the decay term wd * W in fp32 (wd = 0 leaves it as it is, bit for bit: weights are finite)
+    a[e] = __builtin_fmaf(wd, wv4[e], WT == W_BF16 ? bf16_rt(a[e]) : a[e]);
+    const float g = a[e];
     t[e] = __builtin_fmaf(-lr, g, head ? wv4[e] + kv[e] : wv4[e]);
     if (MODE == ROUND_SR_PHILOX) {
       const unsigned r = philox_word0(off0 + (unsigned)e, seed, 0u);
@@ -740,7 +743,7 @@ constexpr int tup_lds_bytes(int halves) { return halves * tup_xbytes(halves); }
 // branches around the products the compiler issued every LDS operand read right in front of its matrix instruction.
 template <int WT, int MODE, int HALVES, bool KAHAN>
 __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES == 2 ? 2 : 1) void tiled_update_kernel(
-    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, TiledSeeds seeds,
+    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, float wd, TiledSeeds seeds,
     int cs, int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
     int red_nchunks, int red_spc, int red_range, int red_bound, int red_round_bf16, float* red_total) {
   static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
@@ -867,7 +870,7 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         const int wq = WT == W_BF16 ? 2 * q : q, kq = kahan_type == 1 ? 2 * q : q;
-        t_update4<WT, MODE>(acc[q], wr + wq, kr + kq, head, kahan_type, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
+        t_update4<WT, MODE>(acc[q], wr + wq, kr + kq, head, kahan_type, lr, wd, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
                             (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * q) >> 2), seed, saturate, wo + wq,
                             ko + kq);
       }
@@ -901,7 +904,7 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
 constexpr int TU2_GBUF = 32768;   // one tile's G: [half][row block][K step] blocks of 1 KiB
 template <int MODE>
 __global__ __launch_bounds__(256, 2) void tiled_update2_kernel(
-    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half, const bf16x8* xt2, float lr, TiledSeeds seeds, int cs,
+    void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half, const bf16x8* xt2, float lr, float wd, TiledSeeds seeds, int cs,
     int saturate, unsigned label0, const floatx4* red_partial, size_t red_part_half, int red_nchunks, int red_spc, int red_range,
     int red_bound, float* red_total) {
   constexpr int RED_BLOCKS = TRED_WAVES * 2 / 4;
@@ -1000,7 +1003,7 @@ __global__ __launch_bounds__(256, 2) void tiled_update2_kernel(
         unsigned wo[3];
 #pragma unroll
         for (int cg = 0; cg < 3; cg++)
-          t_update4<W_E4M3, MODE>(a[cg], &wc[rb][cg], nullptr, false, 0, lr, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * cg),
+          t_update4<W_E4M3, MODE>(a[cg], &wc[rb][cg], nullptr, false, 0, lr, wd, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * cg),
                                   (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * cg) >> 2), seed, saturate, &wo[cg],
                                   nullptr);
         unsigned* dst = (unsigned*)((unsigned char*)w + (size_t)row * D + col0);

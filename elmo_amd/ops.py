@@ -41,9 +41,11 @@ def alloc_workspace(num_chunks, rows_per_chunk, device):
 
 
 def fp8_step(chunks, x, labels, lr, seeds=None, round_mode="rtn", scale_w=1.0, scale_x=1.0, workspace=None,
-             grad_out=None, want_f32=False):
+             grad_out=None, want_f32=False, weight_decay=0.0, dropout_p=0.0, dropout_seed=0):
     """One fused training step (reference: chunked_fp8xmc_clf.py:81-123).  Updates `chunks` in place and returns
-    grad_input (bf16 [B, 768]) or (grad_input, grad_x_fp32) when want_f32."""
+    grad_input (bf16 [B, 768]) or (grad_input, grad_x_fp32) when want_f32.  weight_decay, dropout_p, dropout_seed: the
+    additions of xmc_fp8_step_ex (decay inside the update, dropout of the embedding inside the step); zero = the
+    reference's step."""
     lib = _lib.load()
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2
     assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
@@ -59,10 +61,17 @@ def fp8_step(chunks, x, labels, lr, seeds=None, round_mode="rtn", scale_w=1.0, s
     sarr = None
     if seeds is not None:
         sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
-    st = lib.xmc_fp8_step(arr, nc, rows, x.data_ptr(), batch, feat, labels.data_ptr() if labels.numel() else None,
-                          labels.shape[0], float(lr), sarr, _lib.ROUND_MODES[round_mode], float(scale_w),
-                          float(scale_x), grad_out.data_ptr(), gf.data_ptr() if gf is not None else None,
-                          workspace.data_ptr(), workspace.numel(), _stream_ptr())
+    if weight_decay == 0.0 and dropout_p == 0.0:
+        st = lib.xmc_fp8_step(arr, nc, rows, x.data_ptr(), batch, feat, labels.data_ptr() if labels.numel() else None,
+                              labels.shape[0], float(lr), sarr, _lib.ROUND_MODES[round_mode], float(scale_w),
+                              float(scale_x), grad_out.data_ptr(), gf.data_ptr() if gf is not None else None,
+                              workspace.data_ptr(), workspace.numel(), _stream_ptr())
+    else:
+        st = lib.xmc_fp8_step_ex(arr, nc, rows, x.data_ptr(), batch, feat, labels.data_ptr() if labels.numel() else None,
+                                 labels.shape[0], float(lr), sarr, _lib.ROUND_MODES[round_mode], float(scale_w),
+                                 float(scale_x), float(weight_decay), float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF,
+                                 grad_out.data_ptr(), gf.data_ptr() if gf is not None else None,
+                                 workspace.data_ptr(), workspace.numel(), _stream_ptr())
     _lib.check(st, "xmc_fp8_step")
     return (grad_out, gf) if want_f32 else grad_out
 
@@ -213,7 +222,8 @@ def alloc_tiled_workspace(num_chunks, rows_per_chunk, device, max_batch=MAX_BATC
 
 
 def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=None, round_mode="rtn", workspace=None,
-               grad_out=None, want_f32=False, quantize_x=False, saturate=False, kahan=None, num_head=0, loss_out=None):
+               grad_out=None, want_f32=False, quantize_x=False, saturate=False, kahan=None, num_head=0, loss_out=None,
+               weight_decay=0.0, dropout_p=0.0, dropout_seed=0):
     """One training step of the bf16 layer (chunked.py:76-133) or of the simulated-FP8 mode of the FP8 layer
     (chunked_fp8xmc_clf.py:98-99,110,115-116), three kernels per chunk.  `chunk_views` are contiguous [rows, 768]
     tensors (views of one weight tensor, or the FP8 layer's chunk parameters): all have rows_per_chunk rows except the
@@ -222,7 +232,7 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
     the simulated one; `kahan` ([num_head, 768] bf16 or float8_e5m2, updated in place) turns on the head-Kahan update of
     the first num_head rows of chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127-131).  `loss_out` (a float32 device tensor
     with one element) receives the summed binary cross entropy of the step's logits (what chunked.py:57-72 is written
-    to compute)."""
+    to compute).  weight_decay, dropout_p, dropout_seed: as in fp8_step."""
     lib = _lib.load()
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == FEATURES
     ktype = 0
@@ -253,10 +263,11 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
         sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
     if loss_out is not None:
         assert loss_out.is_cuda and loss_out.dtype == torch.float32 and loss_out.numel() == 1
-    st = lib.xmc_tiled_step(arr, nc, rows_per_chunk, chunk_views[-1].shape[0], WEIGHT_TYPES[weight_type], x.data_ptr(),
+    st = lib.xmc_tiled_step_ex(arr, nc, rows_per_chunk, chunk_views[-1].shape[0], WEIGHT_TYPES[weight_type], x.data_ptr(),
                             batch, FEATURES, labels.data_ptr() if labels.numel() else None, labels.shape[0], float(lr),
                             sarr, _lib.ROUND_MODES[round_mode], int(bool(quantize_x)), int(bool(saturate)),
-                            kahan.data_ptr() if kahan is not None else None, ktype, int(num_head), grad_out.data_ptr(),
+                            kahan.data_ptr() if kahan is not None else None, ktype, int(num_head), float(weight_decay),
+                            float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, grad_out.data_ptr(),
                             gf.data_ptr() if gf is not None else None,
                             loss_out.data_ptr() if loss_out is not None else None, workspace.data_ptr(), workspace.numel(),
                             _stream_ptr())

@@ -16,6 +16,11 @@ Optional, not in the reference (all default to the reference's behaviour):
         sr_fast rounds stochastically with the hardware converter and a counter hash: unbiased on the whole
         e4m3 grid (subnormals included), not bit-identical to the reference's random stream
   training.xmc.scale_w, training.xmc.scale_x   per-tensor scales (reference: 1.0, 1.0)
+  training.xmc.fp8_weight_decay   decay inside the FP8 update, T = W - lr (A + wd W) (reference: none, 0.0)
+  training.xmc.fused_dropout      dropout probability of the embedding applied inside the step while the module is in
+        training mode, in place of an nn.Dropout in front of the layer (model.py:135,165); grad_input is then the
+        gradient in front of that dropout (reference: none, 0.0).  The mask's seed is drawn from the global CPU generator
+        after the chunk seeds.
 """
 import torch
 from torch import nn
@@ -73,6 +78,9 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         assert self.rounding in (("sr_philox", "rtn") if self.fake_fp8_matmul else ("sr_fast", "sr_philox", "rtn"))
         self.scale_w = float(_opt(cfg.training.xmc, "scale_w", 1.0))
         self.scale_x = float(_opt(cfg.training.xmc, "scale_x", 1.0))
+        self.weight_decay = float(_opt(cfg.training.xmc, "fp8_weight_decay", 0.0))
+        self.fused_dropout = float(_opt(cfg.training.xmc, "fused_dropout", 0.0))
+        assert self.weight_decay >= 0.0 and 0.0 <= self.fused_dropout < 1.0
         self.block_size = 16
         self.loss = torch.tensor(0.0, device=self.device)
         self.iteration = 0
@@ -169,20 +177,23 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         loss = 0
         # one seed per chunk from the global CPU generator, exactly as the reference draws them (:113)
         seeds = [torch.randint(0, 1000000, (1,)).item() for _ in range(self.num_chunks)]
+        extra = dict(weight_decay=self.weight_decay)
+        if self.fused_dropout > 0.0 and self.training:
+            extra.update(dropout_p=self.fused_dropout, dropout_seed=torch.randint(0, 2 ** 62, (1,)).item())
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
-                                             round_mode=self.rounding, workspace=self._tiled_workspace)
+                                             round_mode=self.rounding, workspace=self._tiled_workspace, **extra)
         elif embed.shape[0] > ops.MAX_BATCH:
             # the fused kernel holds 128 batch rows; larger batches take the three-kernel path with the same arithmetic
             # (logits from e4m3(X), saturating cast) and the same rounding modes and random words
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128"
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
-                                             saturate=True)
+                                             saturate=True, **extra)
         else:
             self._check_previous_steps()
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
-                                           scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace)
+                                           scale_w=self.scale_w, scale_x=self.scale_x, workspace=self._workspace, **extra)
             self._fused_ran = True
             # the sticky error word follows the step on the stream into pinned host memory; nobody waits for it here
             slot = self._err_next

@@ -77,6 +77,22 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
                  float scale_w, float scale_x, void* grad_x_bf16, float* grad_x_f32, void* workspace,
                  size_t workspace_bytes, void* stream);
 
+/* xmc_fp8_step with three more arguments (no counterpart in the reference's FP8 layer, whose kernels take neither):
+ *   weight_decay  T = W - lr (A + weight_decay * W) in fp32 before the rounding: the decay the reference applies to fp32 /
+ *                 fp16 weights (chunked.py:122-124) and accepts but ignores for low-precision ones
+ *                 (stochastic_rounding_kernel.py:91-99).  0 = xmc_fp8_step.
+ *   dropout_p, dropout_seed
+ *                 dropout of the embedding inside the step (prototype in the reference: src/triton_kernels/tma_gemm.py:7-13,
+ *                 34-38): element (b, k) is kept when tl.rand(dropout_seed, b * 768 + k) > dropout_p, X' = bf16(keep ? X /
+ *                 (1 - p) : 0); logits, grad_W and the update use X' (the logits' operand is e4m3(X' / scale_x)), and
+ *                 grad_x is the gradient with respect to X: (dL/dX') * keep / (1 - p).  The same result as a dropout
+ *                 layer with this mask in front of xmc_fp8_step, without its launches.  dropout_p = 0: xmc_fp8_step.
+ * Everything else as xmc_fp8_step, bit for bit when the three are zero. */
+int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                    int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                    float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
+                    void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Inference logits (chunked_fp8xmc_clf.py:45-60): out[b, label] = bf16(scale * sum_k e4m3(X/scale_x)[b,k] * W[label,k])
  * for label < num_labels (the padding rows of the last chunk are dropped, :60).
  *   out_bf16        device [batch, out_stride] bf16, out_stride >= num_labels; any alignment works, rows that start
@@ -189,6 +205,15 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
                    const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
                    int num_head, void* grad_x_bf16, float* grad_x_f32, float* loss_out, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/* xmc_tiled_step with weight decay and dropout of the embedding, defined as for xmc_fp8_step_ex (for bf16 weights the
+ * decay term joins the bf16-rounded gradient in fp32: T = W - lr (bf16(A) + weight_decay * W)).  With a head-Kahan
+ * buffer (kahan_type != 0) both must be zero, as in the reference's layer: XMC_ERR_MODE otherwise. */
+int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                      const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
+                      const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                      int num_head, float weight_decay, float dropout_p, unsigned long long dropout_seed, void* grad_x_bf16,
+                      float* grad_x_f32, float* loss_out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Measurement aid (no counterpart in the reference): copies `bytes` (a multiple of 16) from src to dst with a plain
  * grid-stride kernel.  Memory-traffic counters are calibrated against this launch of known size. */

@@ -181,6 +181,25 @@ def dropout_quantize(x, p, seed, row_stride=None):
     return e4m3_encode(np.where(keep, scaled, np.float32(0.0)), saturate=True)
 
 
+def dropout_bf16(x, p, seed):
+    """The dropped-out embedding of the steps' fused dropout, in the layer's type: element (b, k) of the bf16-valued fp32
+    array x [B, K] is kept when tl_rand(seed, b * K + k) > p; X' = bf16(keep ? x / (1 - p) : 0) with the division in
+    fp32.  Returns (X' as bf16-valued fp32, keep mask).  Not in the reference's step (its training loop applies
+    nn.Dropout before the layer, model.py:135,165; the prototype of the fusion is tma_gemm.py:7-13)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    offs = (np.arange(m, dtype=np.int64)[:, None] * k + np.arange(k, dtype=np.int64)[None, :])
+    keep = tl_rand(seed, offs) > np.float32(p)
+    scaled = (x / (np.float32(1.0) - np.float32(p))).astype(np.float32)
+    return bf16_round(np.where(keep, scaled, np.float32(0.0)).astype(np.float32)), keep
+
+
+def dropout_backward(g, keep, p):
+    """Gradient in front of the dropout: g * keep / (1 - p), the division in fp32."""
+    g = np.ascontiguousarray(g, dtype=np.float32)
+    return np.where(keep, (g / (np.float32(1.0) - np.float32(p))).astype(np.float32), np.float32(0.0)).astype(np.float32)
+
+
 # --------------------------------------------------------------------------- stochastic rounding
 def sr_add_mask(t, rand, k):
     """The reference bit recipe: add the low k random bits to the fp32 bit pattern, clear the low k bits.

@@ -47,7 +47,7 @@ def _grad_from_logits(z_f32, posmask):
 
 
 def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulated=False,
-             scale_w=1.0, scale_x=1.0, rand_fn=None, return_parts=False):
+             scale_w=1.0, scale_x=1.0, rand_fn=None, return_parts=False, weight_decay=0.0, dropout_p=0.0, dropout_seed=0):
     """One step of the FP8 layer.
 
     w_codes : list of uint8 arrays [L_c, d] (e4m3fn codes), one per chunk (equal L_c)
@@ -60,9 +60,15 @@ def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulate
               bf16 temporary, torch cast back (NaN above 464).
     scale_w, scale_x: per-tensor scales (the reference fixes both at 1.0, :101-102): true weight =
               scale_w * code value, Xq = e4m3(X / scale_x).
+    weight_decay, dropout_p, dropout_seed: this build's additions to the step (xmc_fp8_step_ex), not in the reference's
+              FP8 layer: T = W - lr (A + weight_decay W) with the decayed gradient formed first, in fp32; the step runs
+              on X' = codecs.dropout_bf16(X) and returns the gradient in front of the dropout.
     Returns (new_codes list, gx_fp32 [B,d], grad_input bf16-valued fp32 [B,d]).
     """
     x = np.ascontiguousarray(x_bf16, dtype=np.float32)
+    keep = None
+    if dropout_p > 0:
+        x, keep = C.dropout_bf16(x, dropout_p, dropout_seed)
     B, d = x.shape
     nc = len(w_codes)
     Lc = w_codes[0].shape[0]
@@ -88,6 +94,9 @@ def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulate
         # fuse_kernel.py:102-105; evaluated with a single rounding (fused multiply-add): whether the compiled
         # kernel contracts `w - lr*acc` is unspecified and the two differ by at most one fp32 ulp
         lr_eff = np.float32(lr32 / np.float32(scale_w))
+        if weight_decay:    # decayed gradient A + (wd * scale_w) * code: one fused multiply-add in fp32
+            wd_eff = np.float32(np.float32(weight_decay) * np.float32(scale_w))
+            a = (float(wd_eff) * w64 + a.astype(np.float64)).astype(np.float32)
         t = (w64 - float(lr_eff) * a.astype(np.float64)).astype(np.float32)
         offs = (np.arange(Lc, dtype=np.int64)[:, None] * d + np.arange(d, dtype=np.int64)[None, :])
         if sr_mode == "rtn":
@@ -104,6 +113,8 @@ def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulate
         if return_parts:
             parts.append(dict(z=zb, g=g, a=a, t=t))
     gx32 = gx.astype(np.float32)
+    if keep is not None:
+        gx32 = C.dropout_backward(gx32, keep, dropout_p)
     out = (new_codes, gx32, C.bf16_round(gx32))
     return out + (parts,) if return_parts else out
 
@@ -196,18 +207,23 @@ def topk_of_logits(logits_bf16, k):
 
 
 def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rtn", return_parts=False,
-              return_loss=False):
+              return_loss=False, weight_decay=0.0, dropout_p=0.0, dropout_seed=0):
     """One step of the bf16 layer (chunked.py:85-131), weights bf16.
 
     w_bf16 : fp32 array [L, d] holding bf16 values (single tensor, chunk views of ceil(L/nc) rows, last short)
     sr_mode: "rtn"        W' = bf16(f32(W) - lr*f32(A))
              "reference"  W' = SR16(f32(W) - f32(A)*lr; philox(seed_c, flat idx in chunk))  (stochastic_rounding_kernel.py:80-89)
              "fast"       the same T rounded by sr_bf16_fast with the counter-hash words of the FP8 fast mode (not in the reference)
-    Weight decay is ignored exactly as the bf16 path of the reference ignores it (:91-99).
+    The bf16 path of the reference ignores its weight-decay argument (:91-99): weight_decay = 0 is the reference.  With
+    this build's additions (xmc_tiled_step_ex): T = W - lr (bf16(A) + weight_decay W), the decayed gradient formed first
+    in fp32; dropout as in fp8_step.
     Returns (new_w [L,d] bf16-valued fp32, gx_fp32 [B,d], grad_input bf16-valued fp32[, loss with return_loss]).
     """
     w_all = np.ascontiguousarray(w_bf16, dtype=np.float32)
     x = np.ascontiguousarray(x_bf16, dtype=np.float32)
+    keep = None
+    if dropout_p > 0:
+        x, keep = C.dropout_bf16(x, dropout_p, dropout_seed)
     B, d = x.shape
     L = w_all.shape[0]
     cs = (L + num_chunks - 1) // num_chunks
@@ -230,6 +246,8 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
         g64 = g.astype(np.float64)
         gx = gx + C.bf16_round((g64 @ w64).astype(np.float32))      # partial rounded to bf16 (:116)
         a = C.bf16_round((g64.T @ x64).astype(np.float32))          # materialised bf16 grad (:119)
+        if weight_decay:
+            a = (float(np.float32(weight_decay)) * w64 + a.astype(np.float64)).astype(np.float32)
         if sr_mode == "rtn":
             t = (w64 - float(lr32) * a.astype(np.float64)).astype(np.float32)   # single rounding (fma)
             nw = C.bf16_round(t)
@@ -248,6 +266,8 @@ def bf16_step(w_bf16, x_bf16, labels, lr, num_chunks, *, seeds=None, sr_mode="rt
         new_w[lo:hi] = nw
         if return_parts:
             parts.append(dict(z=zb, g=g, a=a, t=t))
+    if keep is not None:
+        gx = C.dropout_backward(gx, keep, dropout_p)
     out = (new_w, gx, C.bf16_round(gx))
     if return_loss:
         out = out + (loss,)

@@ -105,6 +105,42 @@ def test_sampled_rows_match_oracle_after_a_real_step(gpu, big):
     assert np.mean(got != w_old) > 0.3                       # the step really changed the weights
 
 
+def test_sampled_rows_match_exact_stochastic_rounding_after_a_real_sr_fast_step(gpu, big):
+    """The headline's own rounding mode at full size: after a real `sr_fast` step over all 670 K labels, sampled rows
+    (tile and chunk boundaries, labels with positives, random ones) equal the oracle's exact stochastic rounding fed with
+    the same counter-hash words (global row, column, hashed per-chunk seed), up to the one-grid-step differences the fp32
+    summation order of grad_W causes."""
+    import torch
+    from elmo_amd import ops
+    nc, rows = big["nc"], big["rows"]
+    rng = np.random.default_rng(1)
+    pos_rows = np.unique(big["labels_np"][:, 1])
+    sample = np.unique(np.concatenate([np.arange(0, 70), pos_rows[:150], [rows - 1, rows, rows + 63, rows + 64, 5 * rows - 1, nc * rows - 1],
+                                       rng.integers(0, nc * rows, 300)]))
+    seeds = [1000 + 17 * c for c in range(nc)]
+    before = np.stack([big["chunks"][r // rows][r % rows].view(torch.uint8).cpu().numpy().copy() for r in sample])
+    ws = ops.alloc_workspace(nc, rows, gpu)
+    ops.fp8_step(big["chunks"], big["x"], big["labels"], 0.05, seeds=seeds, round_mode="sr_fast", workspace=ws)
+    assert ops.step_error_word(ws, nc, rows) == 0
+    remap = {int(r): i for i, r in enumerate(sample)}
+    lab = np.array([(b, remap[int(l)]) for b, l in big["labels_np"] if int(l) in remap], dtype=np.int32).reshape(-1, 2)
+
+    def rand_fn(c, offs):          # the oracle sees one chunk made of the sampled rows: map its offsets back
+        r, k = offs // 768, offs % 768
+        grow = sample[r]
+        out = np.zeros(offs.shape, dtype=np.uint32)
+        for ch in np.unique(grow // rows):           # the seed is per chunk
+            sel = grow // rows == ch
+            out[sel] = C.fast_sr_words(seeds[int(ch)], grow[sel], k[sel])
+        return out
+
+    ref_codes, _, _ = O.fp8_step([before], big["x_np"], lab, 0.05, sr_mode="exact", rand_fn=rand_fn)
+    got = np.stack([big["chunks"][r // rows][r % rows].view(torch.uint8).cpu().numpy() for r in sample])
+    d = H.e4m3_ulp_distance(got, ref_codes[0])
+    assert d.max() <= 1 and np.mean(d != 0) < 2e-3
+    assert np.mean(got != before) > 0.3
+
+
 def test_batch_256_at_the_chunk_size_of_the_largest_workload(gpu):
     """True FP8 with 256 batch rows on chunks of 262,144 rows (the chunk size of the 8.6 M-label workload, four chunks
     here): the one-pass FP8 logits, the eight-wavefront grad_X and the feature-split update at their real launch shapes.

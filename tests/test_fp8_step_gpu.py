@@ -13,7 +13,7 @@ from oracle import step as O
 pytestmark = pytest.mark.gpu
 
 
-def run_rtn(case, device, lr=0.05, scale_w=1.0, scale_x=1.0, device_labels=None):
+def run_rtn(case, device, lr=0.05, scale_w=1.0, scale_x=1.0, device_labels=None, **extra):
     import torch
     from elmo_amd import ops
     chunks, x, labels = H.to_device_case(case, device)
@@ -21,11 +21,11 @@ def run_rtn(case, device, lr=0.05, scale_w=1.0, scale_x=1.0, device_labels=None)
         labels = torch.from_numpy(np.ascontiguousarray(device_labels, dtype=np.int32)).to(device)
     ws = ops.alloc_workspace(len(chunks), chunks[0].shape[0], device)
     g, gf = ops.fp8_step(chunks, x, labels, lr, round_mode="rtn", scale_w=scale_w, scale_x=scale_x, workspace=ws,
-                         want_f32=True)
+                         want_f32=True, **extra)
     assert ops.step_error_word(ws, len(chunks), chunks[0].shape[0]) == 0
     new = H.chunks_to_numpy(chunks)
     ref_codes, ref_gx, ref_gb = O.fp8_step(case["chunks"], case["x"], case["labels"], lr, sr_mode="rtn",
-                                           scale_w=scale_w, scale_x=scale_x)
+                                           scale_w=scale_w, scale_x=scale_x, **extra)
     return new, gf.cpu().numpy(), H.bf16_tensor_to_f32_numpy(g), ref_codes, ref_gx, ref_gb
 
 
@@ -130,6 +130,30 @@ def test_scales(gpu):
     # weights stored as w / 2^-4, so most codes sit in the normal range
     case = H.make_case(2, 512, 32, 33, w_scale=2.0 ** -4)
     check_rtn(case, gpu, scale_w=2.0 ** -4, scale_x=0.5)
+
+
+@pytest.mark.parametrize("wd,p,sw", [(0.05, 0.0, 1.0), (0.0, 0.3, 1.0), (0.02, 0.1, 2.0 ** -4)])
+def test_weight_decay_and_fused_dropout(gpu, wd, p, sw):
+    """T = c - (lr / s)(A + wd s c) and the dropout of X inside the step, against the oracle (which is pinned by closed
+    forms for both).  lr and wd are large enough that the decay term moves a good share of the weights by itself."""
+    import torch
+    from elmo_amd import ops
+    case = H.make_case(3, 1008, 48, 35, w_scale=sw)
+    check_rtn(case, gpu, lr=0.5, scale_w=sw, weight_decay=wd, dropout_p=p, dropout_seed=0xABCDEF0123)
+    plain = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.5, scale_w=sw)
+    extra = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.5, scale_w=sw, weight_decay=wd, dropout_p=p,
+                       dropout_seed=0xABCDEF0123)
+    assert np.mean(np.concatenate(plain[0]) != np.concatenate(extra[0])) > 0.02      # the options matter on this case
+    # the stochastic modes take the same decayed T: the reference's recipe is bit-identical wherever T is
+    chunks, x, labels = H.to_device_case(case, gpu)
+    seeds = [5, 6, 7]
+    ops.fp8_step(chunks, x, labels, 0.5, seeds=seeds, round_mode="sr_philox", scale_w=sw, weight_decay=wd, dropout_p=p,
+                 dropout_seed=0xABCDEF0123)
+    ref = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.5, seeds=seeds, sr_mode="reference", scale_w=sw,
+                     weight_decay=wd, dropout_p=p, dropout_seed=0xABCDEF0123)[0]
+    got = H.chunks_to_numpy(chunks)
+    d = np.concatenate([H.e4m3_ulp_distance(a, b).ravel() for a, b in zip(got, ref)])
+    assert d.max() <= 1 and (d != 0).mean() < 2e-3
 
 
 def test_x_not_modified_and_deterministic(gpu):

@@ -72,6 +72,40 @@ def test_training_call_contract(gpu):
     assert np.abs(g.float().cpu().numpy() * 2 - ref_gb).max() <= 2e-2 * np.abs(ref_gb).max()
 
 
+def test_module_options_for_weight_decay_and_fused_dropout(gpu):
+    """training.xmc.fp8_weight_decay and training.xmc.fused_dropout (absent: the reference's behaviour, checked by every
+    other test of this file): the step equals the oracle's with the same options and the seed the module drew from the
+    global CPU generator after the chunk seeds; in eval mode no dropout is applied."""
+    import torch
+    xfc = build(gpu, 1000, 2, rounding="rtn", fp8_weight_decay=0.2, fused_dropout=0.25)
+    before = [w.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    torch.manual_seed(3)
+    x = (0.05 * torch.randn(32, 768, device=gpu)).to(torch.bfloat16)
+    labels = torch.tensor([[0, 3], [0, 999], [5, 17], [31, 500]], dtype=torch.int32, device=gpu)
+    torch.manual_seed(77)
+    xfc.train()
+    xfc.xfc_forward_backward(x, labels, [0.5])
+    torch.manual_seed(77)
+    for _ in range(2):
+        torch.randint(0, 1000000, (1,)).item()
+    dseed = torch.randint(0, 2 ** 62, (1,)).item()
+    ref_codes, ref_gx, ref_gb = O.fp8_step(before, x.float().cpu().numpy(), labels.cpu().numpy(), 0.5, weight_decay=0.2,
+                                           dropout_p=0.25, dropout_seed=dseed)
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        d = H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r)
+        assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    g = xfc.grad_input.float().cpu().numpy()
+    assert np.array_equal(g == 0, ref_gb == 0)                     # the same mask
+    assert np.abs(g - ref_gb).max() <= 2e-2 * np.abs(ref_gb).max()
+    xfc.eval()
+    mid = [w.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    xfc.xfc_forward_backward(x, labels, [0.5])
+    ref_codes = O.fp8_step(mid, x.float().cpu().numpy(), labels.cpu().numpy(), 0.5, weight_decay=0.2)[0]
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        assert H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r).max() <= 1
+    assert xfc.last_step_error() == 0
+
+
 def test_default_rounding_draws_seeds_from_the_global_cpu_generator(gpu):
     import torch
     xfc = build(gpu, 500, 3)

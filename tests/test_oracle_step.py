@@ -251,6 +251,53 @@ def test_kahan_step_invariants():
     assert np.array_equal(c8[0], cb[0]) and np.abs(C.e5m2_decode(k8) - kb).max() <= 2.0 ** -3 * np.abs(kb).max()
 
 
+def test_kahan_update_scalar_evaluation_pins_the_order_of_operations():
+    """The compensated update of the head rows, element by element in fp32 scalars and in the order the reference's
+    kernel writes it (fuse_kernel.py:243-258):
+        weights = weights + kahan;  weights = weights - lr*acc;  weights_new = round(weights)
+        kahan   = kahan + weights_old - weights_new - lr*acc          (left to right)
+    on a case built so that the fp32 sum kahan + weights_old is inexact: another association of the three operations of
+    the second line (kahan + (weights_old - weights_new) - lr*acc, say) gives other buffer values, so the oracle's
+    order is pinned, not just its invariants."""
+    rng = np.random.default_rng(12)
+    d, B, L, num_head = 8, 4, 16, 3
+    w_codes = rng.integers(0x30, 0x48, size=(L, d)).astype(np.uint8)            # weights of magnitude 0.5 .. 4
+    w_codes[::2] |= 0x80
+    # compensation values with bits far below the weights' last fp32 place: 2^-20 * (1 + j/128), stored as bf16
+    kahan = C.bf16_round((2.0 ** -20 * (1.0 + rng.integers(1, 127, size=(num_head, d)) / 128.0)).astype(np.float32))
+    kahan[:, ::3] *= -1
+    x = C.bf16_round(rng.normal(size=(B, d)).astype(np.float32))
+    x[:, :3] = 0.0      # no gradient for these features: there the new buffer value is (kahan + weights_old) - weights_new,
+                        # whose fp32 rounding of the first sum is large enough to survive the cast to bf16
+    labels = np.array([(0, 1), (2, 0)], dtype=np.int32)
+    lr = 0.05
+    new_codes, new_kahan, _, _ = O.fp8_kahan_step([w_codes], kahan, x, labels, lr, num_head, kahan_type="bf16", sr_mode="rtn")
+    # G of the head rows from the oracle's own (separately pinned) forward part
+    _, _, _, parts = O.fp8_step([w_codes], x, labels, lr, return_parts=True)
+    g = parts[0]["g"]
+    lr32 = np.float32(lr)
+    w = C.e4m3_decode(w_codes)
+    differs = 0
+    for l in range(num_head):
+        for f in range(d):
+            acc = np.float32(sum(float(g[l, b]) * float(x[b, f]) for b in range(B)))       # exact in float64, one rounding
+            weights_old = np.float32(w[l, f])
+            k = np.float32(kahan[l, f])
+            weights = np.float32(weights_old + k)                                           # weights + kahan
+            weights = np.float32(np.float64(weights) - np.float64(lr32) * np.float64(acc))  # - lr*acc (fused)
+            code = C.e4m3_encode(np.array([weights], dtype=np.float32), saturate=True)[0]
+            weights_new = np.float32(C.e4m3_decode(np.array([code], dtype=np.uint8))[0])
+            t1 = np.float32(k + weights_old)                                                # kahan + weights_old
+            t2 = np.float32(t1 - weights_new)                                               # - weights_new
+            kn = np.float32(np.float64(t2) - np.float64(lr32) * np.float64(acc))            # - lr*acc (fused)
+            assert code == new_codes[0][l, f]
+            assert C.bf16_round(np.array([kn], dtype=np.float32))[0] == new_kahan[l, f], (l, f)
+            # the other association: kahan + (weights_old - weights_new) - lr*acc
+            alt = np.float32(np.float64(np.float32(k + np.float32(weights_old - weights_new))) - np.float64(lr32) * np.float64(acc))
+            differs += int(C.bf16_round(np.array([alt], dtype=np.float32))[0] != new_kahan[l, f])
+    assert differs > 0, "the case does not distinguish the orders of operations"
+
+
 def test_loss_matches_the_library_routine_and_the_cited_op_sequence():
     """bce_loss_sum against torch's binary_cross_entropy_with_logits (float64, sum) and against the operations of
     chunked.py:61-72 restated one by one in fp32; and the step's loss against the same routine on the oracle's logits."""
@@ -343,3 +390,76 @@ def test_dense_step_matches_torch_cpu(dtype, tdt):
     # weight decay is in effect: the same step without it ends elsewhere
     no_wd, _, _ = O.dense_step(w, x, labels, lr, 0.0, nc, dtype)
     assert np.abs(no_wd - new).max() > 10 * ulp * np.abs(new).max()
+
+
+def _e4m3_half_spacing(v):
+    """Half the distance between neighbouring e4m3 values around v (normal binades carry 3 mantissa bits; below 2^-6
+    the grid is uniform with spacing 2^-9)."""
+    e = np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -6)))
+    return 2.0 ** (e - 3) / 2
+
+
+def test_weight_decay_closed_forms():
+    """Weight decay inside the low-precision updates (this build's addition; the reference applies decay only to its
+    fp32 / fp16 dense layers).  (1) X = 0 makes the gradient of W vanish, so the step reduces to
+    T = c - (lr / s) f32(wd s c) on the codes c: checked against torch's CPU casts, with and without a weight scale.
+    (2) On a general case the new codes are the nearest e4m3 values of c - (lr / s)(A + wd s c) evaluated in float64
+    from the oracle's own gradient A: a dropped term, a wrong sign or a misplaced scale moves them by whole steps."""
+    w, x, labels = tiny_case(L=24, d=16, B=4, seed=5)
+    wt = torch.from_numpy(w).view(torch.float8_e4m3fn).float()
+    lr, wd = 0.5, 0.125
+    for s in (1.0, 0.25):
+        new, gx, _ = O.fp8_step([w], np.zeros_like(x), labels, lr, scale_w=s, weight_decay=wd)
+        lr_eff = torch.tensor(lr, dtype=torch.float32) / torch.tensor(s, dtype=torch.float32)
+        g = (torch.tensor(wd * s, dtype=torch.float32) * wt)
+        want = (wt - lr_eff * g).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        assert np.array_equal(new[0], want)
+        assert not np.array_equal(new[0], w)
+    # bf16 layer, X = 0
+    wb = C.bf16_round(np.random.default_rng(2).standard_normal((24, 16)).astype(np.float32))
+    newb, _, _ = O.bf16_step(wb, np.zeros_like(x), labels, lr, 2, weight_decay=wd)
+    wbt = torch.from_numpy(wb)
+    wantb = (wbt - torch.tensor(lr) * (torch.tensor(wd) * wbt)).bfloat16().float().numpy()
+    assert np.array_equal(newb, wantb)
+    # general case
+    for s in (1.0, 0.5):
+        new0, _, _, parts0 = O.fp8_step([w], x, labels, lr, scale_w=s, return_parts=True)
+        new1, gx1, _ = O.fp8_step([w], x, labels, lr, scale_w=s, weight_decay=wd)
+        a = parts0[0]["a"].astype(np.float64)                       # the gradient without decay
+        c = C.e4m3_decode(w).astype(np.float64)
+        t64 = np.clip(c - (lr / s) * (a + wd * s * c), -448, 448)
+        got = C.e4m3_decode(new1[0]).astype(np.float64)
+        assert np.all(np.abs(got - t64) <= _e4m3_half_spacing(t64) * (1 + 1e-3) + 1e-9)
+        assert not np.array_equal(new0[0], new1[0])
+        # decay does not enter the gradient of X
+        assert np.array_equal(gx1, O.fp8_step([w], x, labels, lr, scale_w=s)[1])
+    # zero decay is the reference's update, bit for bit
+    assert np.array_equal(O.fp8_step([w], x, labels, lr, weight_decay=0.0)[0][0], O.fp8_step([w], x, labels, lr)[0][0])
+
+
+def test_fused_dropout_is_a_dropout_layer_in_front_of_the_step():
+    """Dropout of the embedding inside the step (this build's addition; the reference's loop applies nn.Dropout before
+    the layer, model.py:135,165): the step on X with (p, seed) equals the plain step on X' = bf16(keep ? X / (1 - p) : 0)
+    with X' built by torch on the CPU from the Triton-pinned uniform numbers, and its grad_x is the plain step's gradient
+    passed back through the mask.  About (1 - p) of the elements survive; p = 0 changes nothing."""
+    w, x, labels = tiny_case(L=24, d=16, B=4, seed=8)
+    p, seed = 0.3, 0x1234_5678_9ABC
+    offs = np.arange(x.size, dtype=np.int64).reshape(x.shape)
+    keep = torch.from_numpy(C.tl_rand(seed, offs) > np.float32(p))
+    xt = torch.from_numpy(x)
+    xd = torch.where(keep, xt / (torch.tensor(1.0) - torch.tensor(p, dtype=torch.float32)), torch.zeros(())).bfloat16().float()
+    assert 0 < int(keep.sum()) < x.size
+    for fn, args in ((O.fp8_step, ([w], x, labels, 0.05)), (O.bf16_step, (C.e4m3_decode(w), x, labels, 0.05, 2))):
+        a2 = list(args); a2[1] = xd.numpy()
+        plain = fn(*a2)
+        fused = fn(*args, dropout_p=p, dropout_seed=seed)
+        assert np.array_equal(np.asarray(plain[0]), np.asarray(fused[0]))
+        back = torch.where(keep, torch.from_numpy(plain[1]) / (torch.tensor(1.0) - torch.tensor(p, dtype=torch.float32)),
+                           torch.zeros(())).numpy()
+        assert np.array_equal(fused[1], back)
+        assert np.array_equal(fused[2], C.bf16_round(back))
+        same = fn(*args, dropout_p=0.0, dropout_seed=seed)
+        ref = fn(*args)
+        assert np.array_equal(np.asarray(same[0]), np.asarray(ref[0])) and np.array_equal(same[1], ref[1])
+    big = C.tl_rand(7, np.arange(1 << 16)) > np.float32(p)
+    assert abs(big.mean() - (1 - p)) < 0.01

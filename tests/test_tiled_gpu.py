@@ -74,6 +74,45 @@ def test_bf16_layer_rtn_parity(gpu, L, nc, batch, seed):
     check_gx(gf, gb, ref_gx, tol=4e-3)
 
 
+@pytest.mark.parametrize("wd,p", [(0.05, 0.0), (0.0, 0.3), (0.02, 0.1)])
+def test_weight_decay_and_fused_dropout_on_the_three_kernel_path(gpu, wd, p):
+    """bf16 layer: T = W - lr (bf16(A) + wd W) and dropout of X in the preparation kernel; simulated-FP8 mode: the same
+    with the fp32 gradient.  Against the oracle, whose treatment of both is pinned by closed forms on the CPU."""
+    import torch
+    from elmo_amd import ops
+    L, nc, batch, lr, dseed = 3000, 3, 40, 0.5, 0x1357_9BDF_2468
+    x, w, labels = bf16_case(L, batch, 39)
+    cs = (L + nc - 1) // nc
+    wt = torch.from_numpy(C.bf16_bits(w).view(np.int16)).to(gpu).view(torch.bfloat16)
+    views = [wt[c * cs:min((c + 1) * cs, L)] for c in range(nc)]
+    xt = torch.from_numpy(C.bf16_bits(x).view(np.int16)).to(gpu).view(torch.bfloat16)
+    lab = torch.from_numpy(labels).to(gpu).contiguous()
+    g, gf = ops.tiled_step(views, cs, "bf16", xt, lab, lr, want_f32=True, weight_decay=wd, dropout_p=p, dropout_seed=dseed)
+    ref_w, ref_gx, _ = O.bf16_step(w, x, labels, lr, nc, weight_decay=wd, dropout_p=p, dropout_seed=dseed)
+    plain_w = O.bf16_step(w, x, labels, lr, nc)[0]
+    assert (plain_w != ref_w).mean() > 0.02
+    check_bf16_weights(wt.float().cpu().numpy(), ref_w, w, x, lr=lr)
+    check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx, tol=4e-3)
+    if p > 0:       # dropped elements have an exactly zero gradient
+        keep = C.dropout_bf16(x, p, dseed)[1]
+        assert np.all(gf.cpu().numpy()[~keep] == 0) and np.any(gf.cpu().numpy()[keep] != 0)
+    # simulated FP8
+    case = H.make_case(3, 1008, 48, 64)
+    chunks, xs, labs = H.to_device_case(case, gpu)
+    g, gf = ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", xs, labs, lr, want_f32=True, weight_decay=wd, dropout_p=p,
+                           dropout_seed=dseed)
+    ref_codes, ref_gx, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], lr, simulated=True, weight_decay=wd,
+                                      dropout_p=p, dropout_seed=dseed)
+    d = np.concatenate([H.e4m3_ulp_distance(a, b).ravel() for a, b in zip(H.chunks_to_numpy(chunks), ref_codes)])
+    assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    check_gx(gf.cpu().numpy(), g.float().cpu().numpy(), ref_gx)
+    # the head-Kahan layer takes neither option
+    kah = torch.zeros(64, 768, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(Exception):
+        ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", xs, labs, lr, quantize_x=True, saturate=True, kahan=kah,
+                       num_head=64, weight_decay=0.01)
+
+
 def test_bf16_layer_reference_stochastic_rounding(gpu):
     L, nc, batch = 3000, 3, 32
     x, w, labels = bf16_case(L, batch, 41)
