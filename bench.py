@@ -268,6 +268,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=100.0,
                     help="milliseconds of device conditioning before the warm-up steps (the fused step on a separate classifier of the same shape); 0 = none")
+    ap.add_argument("--head-kahan", default="none", choices=["none", "bf16", "e5m2"],
+                    help="time the head-Kahan layer's fused step instead (fused workloads only): compensation buffer of "
+                         "this type on the first min(head_ratio x padded labels, rows per chunk) rows of chunk 0")
+    ap.add_argument("--head-ratio", type=float, default=0.2, help="training.FP8.head_ratio of the reference's configs")
     ap.add_argument("--scale-w", type=float, default=1.0,
                     help="per-tensor scale of the weights (weight = scale_w * code); the reference uses 1")
     ap.add_argument("--scale-x", type=float, default=1.0, help="per-tensor scale of the quantised embedding")
@@ -337,8 +341,21 @@ def main():
     grad = torch.empty(cfg.batch, cfg.dim, dtype=torch.bfloat16, device=dev)
     seed_rng = np.random.default_rng(cfg.seed)
 
+    num_head, kahan = 0, None
+    if args.head_kahan != "none":
+        # the reference requires head_ratio x labels <= rows per chunk (chunked_head_kahan_fp8xmc_clf.py:48); the workload's
+        # chunking is kept here and the head is cut at the first chunk's end
+        assert args.scale_w == 1.0 and args.scale_x == 1.0, "the head-Kahan layer has no per-tensor scales"
+        num_head = min(int(args.head_ratio * L_pad), rows)
+        kahan = torch.zeros(num_head, cfg.dim, dtype=torch.bfloat16 if args.head_kahan == "bf16" else torch.float8_e5m2,
+                            device=dev)
+
     def one_step():
         seeds = seed_rng.integers(0, 1_000_000, size=nc)
+        if kahan is not None:
+            ops.fp8_kahan_step(chunks, kahan, num_head, x, labels, cfg.lr, seeds=seeds, round_mode=args.round,
+                               workspace=workspace, grad_out=grad)
+            return
         ops.fp8_step(chunks, x, labels, cfg.lr, seeds=seeds, round_mode=args.round, scale_w=args.scale_w, scale_x=args.scale_x,
                      workspace=workspace, grad_out=grad)
 
@@ -409,7 +426,8 @@ def main():
     modes = {args.round: {"steps_per_s": args.steps / elapsed, "ms_per_step": elapsed / args.steps * 1e3, "kernel_ms": kernel_ms,
                           "roofline_frac_kernel": 2.0 * cfg.num_labels * cfg.dim / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}}
     other = "sr_philox" if args.round != "sr_philox" else "sr_fast"
-    modes[other] = timed_mode(other, min(args.steps, 40))
+    if kahan is None:
+        modes[other] = timed_mode(other, min(args.steps, 40))
     ms_per_step = elapsed / args.steps * 1e3
     steps_per_s = args.steps / elapsed
     peak_bytes = torch.cuda.max_memory_allocated() - base_alloc + weight_bytes
@@ -435,7 +453,8 @@ def main():
         "dtype": "fp8_e4m3 weights+logits MFMA, bf16 gradient MFMA, fp32 accumulate", "data": "synthetic",
         "config": {"workload": cfg.name, "labels": cfg.num_labels, "labels_padded": L_pad, "features": cfg.dim,
                    "batch": cfg.batch, "chunks": nc, "rows_per_chunk": rows, "positives": int(labels.shape[0]),
-                   "lr": cfg.lr, "rounding": args.round, "seed": cfg.seed, "scale_w": args.scale_w, "scale_x": args.scale_x},
+                   "lr": cfg.lr, "rounding": args.round, "seed": cfg.seed, "scale_w": args.scale_w, "scale_x": args.scale_x,
+                   "head_kahan": args.head_kahan, "num_head": num_head},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "traffic_source": "carried over, not measured in this run: profiles/hbm_traffic.json holds rocprofv3 --pmc "

@@ -51,6 +51,9 @@ def load():
     lib.xmc_fp8_step_ex.restype = i32
     lib.xmc_fp8_step_ex.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, vp, i32, f32,
                                     ctypes.POINTER(ctypes.c_uint32), i32, f32, f32, f32, f32, ctypes.c_ulonglong, vp, vp, vp, sz, vp]
+    lib.xmc_fp8_kahan_step.restype = i32
+    lib.xmc_fp8_kahan_step.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, vp, i32, f32,
+                                       ctypes.POINTER(ctypes.c_uint32), i32, vp, i32, i32, vp, vp, vp, sz, vp]
     lib.xmc_fp8_forward.restype = i32
     lib.xmc_fp8_forward.argtypes = [ctypes.POINTER(vp), i32, i32, vp, i32, i32, f32, f32, vp, ll, ll, vp, sz, vp]
     lib.xmc_fp8_forward_static.restype = i32

@@ -6,10 +6,15 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "csrc", "xmc_capi.hip")
 OUT = os.path.join(HERE, "libelmo_xmc.so")
 
+SRC_HEAVY = os.path.join(HERE, "csrc", "xmc_fp8_role_heavy.hip")
+
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-munsafe-fp-atomics",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# The second translation unit holds the variants of the step kernel whose tile loop is too large for the compiler's
+# default "#pragma unroll" size limit (see the head of that file); everything else keeps the default.
+HEAVY_FLAGS = ["-mllvm", "-pragma-unroll-threshold=1000000"]
 
 
 def source_files():
@@ -44,19 +49,30 @@ def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     digest = source_hash()
     tmp = OUT + ".tmp%d" % os.getpid()
-    cmd = [hipcc] + HIPCC_FLAGS + [f'-DXMC_SOURCE_HASH="{digest}"', SRC, "-o", tmp]
-    if verbose:
-        cmd.append("-Rpass-analysis=kernel-resource-usage")
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        if os.path.exists(tmp):
-            os.remove(tmp)
-        raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+    extra = ["-Rpass-analysis=kernel-resource-usage"] if verbose else []
+    objs = [tmp + ".main.o", tmp + ".heavy.o"]
+    cmds = [[hipcc] + HIPCC_FLAGS + extra + [f'-DXMC_SOURCE_HASH="{digest}"', "-c", SRC, "-o", objs[0]],
+            [hipcc] + HIPCC_FLAGS + HEAVY_FLAGS + extra + ["-c", SRC_HEAVY, "-o", objs[1]]]
+    procs = [subprocess.Popen(c, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True) for c in cmds]   # side by side
+    outs = [p.communicate() for p in procs]
+    log = "".join(o[0] + o[1] for o in outs)
+    try:
+        if any(p.returncode != 0 for p in procs):
+            raise RuntimeError("hipcc failed:\n" + log)
+        res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", tmp], capture_output=True, text=True)
+        if res.returncode != 0:
+            if os.path.exists(tmp):
+                os.remove(tmp)
+            raise RuntimeError("hipcc (link) failed:\n" + res.stdout + res.stderr)
+    finally:
+        for o in objs:
+            if os.path.exists(o):
+                os.remove(o)
     # moved into place in one step: a process that has the previous library mapped keeps its (unlinked) file
     os.replace(tmp, OUT)
     with open(HASH_FILE, "w") as f:
         f.write(digest + "\n")
-    return res.stderr if verbose else OUT
+    return log if verbose else OUT
 
 
 def ensure_built():

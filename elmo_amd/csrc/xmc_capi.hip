@@ -40,12 +40,11 @@ void fill_device_info(int dev) {
   void* sp = nullptr;
   di.scratch_ptr = (di.ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess) ? (unsigned char*)sp : nullptr;
   // opt in to the full 160 KiB of LDS once per device
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_RTN, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_PHILOX, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST, false>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<ROUND_SR_FAST, true>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES);
+#define XMC_STEP_LDS(RMODE, WD) \
+  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<RMODE, WD, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES)
+  XMC_STEP_LDS(ROUND_RTN, false); XMC_STEP_LDS(ROUND_RTN, true); XMC_STEP_LDS(ROUND_SR_FAST, false); XMC_STEP_LDS(ROUND_SR_FAST, true);
+#undef XMC_STEP_LDS
+  role_heavy_set_lds();
   (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
@@ -176,7 +175,8 @@ size_t xmc_workspace_bytes(int num_chunks, int rows_per_chunk) {
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0) return 0;
   size_t tiles = (size_t)num_chunks * ((rows_per_chunk + TL - 1) / TL);
   // tile_ptr, then 32-byte tile descriptors, one run per quad (up to MAX_WG / 4 runs, each rounded up to whole entries)
-  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256 + (tiles + MAX_WG / 4) * 32;
+  // (two tables with a compensated head)
+  return WS_TILEPTR + ((tiles + 1) * 4 + 255) / 256 * 256 + (tiles + MAX_WG / 2) * 32;
 }
 
 int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
@@ -187,10 +187,14 @@ int xmc_fp8_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
                          scale_w, scale_x, 0.0f, 0.0f, 0ull, grad_x_bf16, grad_x_f32, workspace, workspace_bytes, stream_);
 }
 
-int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
-                    int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
-                    float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
-                    void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream_) {
+}  // extern "C"
+
+// The fused step behind xmc_fp8_step, xmc_fp8_step_ex and xmc_fp8_kahan_step.  kahan_type 0: no compensated head.
+static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                      int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                      float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
+                      void* kahan, int kahan_type, int num_head,
+                      void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream_) {
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
   if (!grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
@@ -200,6 +204,14 @@ int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
   if (!(scale_w > 0.f) || !(scale_x > 0.f)) return XMC_ERR_SHAPE;
   if (!(weight_decay >= 0.f) || !(dropout_p >= 0.f) || !(dropout_p < 1.f)) return XMC_ERR_SHAPE;
+  if (kahan_type < 0 || kahan_type > 2) return XMC_ERR_MODE;
+  if (kahan_type != 0) {
+    if (!kahan) return XMC_ERR_NULL;
+    if (!aligned16(kahan)) return XMC_ERR_ALIGN;
+    if (num_head <= 0 || num_head > rows_per_chunk) return XMC_ERR_SHAPE;
+  } else {
+    num_head = 0;
+  }
   DeviceInfo di = device_info();
   if (di.ok != 1 || di.cus < 16) return XMC_ERR_DEVICE;
   hipStream_t stream = (hipStream_t)stream_;
@@ -222,6 +234,7 @@ int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
     p.rows_per_chunk = rows_per_chunk;
     p.tiles_per_chunk = tiles_per_chunk;
     p.num_tiles = num_tiles;
+    p.run_tiles = num_tiles;
     p.xq = ws + WS_XQ;
     p.xt = (const bf16x8*)(ws + WS_XT);
     p.keys = (const unsigned*)(ws + WS_KEYS);
@@ -241,7 +254,15 @@ int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
 #endif
     if (qgrid < 32) return XMC_ERR_DEVICE;
     p.nquads = qgrid >> 2;
-    p.kmax = (num_tiles + p.nquads - 1) / p.nquads;
+    // with a compensated head the tiles that hold its rows run first, as a launch of their own
+    const int head_tiles = (num_head + TL - 1) / TL, rest_tiles = num_tiles - head_tiles;
+    p.kahan = (unsigned char*)kahan;
+    p.num_head = num_head;
+    p.head_tiles = head_tiles;
+    p.kmax_head = (head_tiles + p.nquads - 1) / p.nquads;
+    p.kmax = (rest_tiles + p.nquads - 1) / p.nquads;
+    p.cnt_base = 0;
+    p.acc_init = 0;
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
         labels_coo, nnz, n_pad, batch, 0, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
@@ -249,23 +270,49 @@ int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
         (unsigned short*)(ws + WS_XT), dp);
     if (g_prof_start) (void)hipEventRecord(g_prof_start, stream);
-#define XMC_LAUNCH_STEP(RMODE)                                                                             \
-  do {                                                                                                     \
-    if (weight_decay != 0.f) fp8_step_role_kernel<RMODE, true><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);     \
-    else fp8_step_role_kernel<RMODE, false><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);                        \
-  } while (0)
-    switch (round_mode) {
-      case XMC_ROUND_RTN: XMC_LAUNCH_STEP(ROUND_RTN); break;
-      case XMC_ROUND_SR_PHILOX: XMC_LAUNCH_STEP(ROUND_SR_PHILOX); break;
-      default: XMC_LAUNCH_STEP(ROUND_SR_FAST); break;
+    QuadParams ph = p;   // the head's launch
+    ph.run_tiles = head_tiles;
+    ph.kmax = p.kmax_head;
+    p.run_tiles = rest_tiles;
+    p.desc = desc + 2 * (size_t)p.nquads * p.kmax_head;
+    if (head_tiles > 0) { p.cnt_base = QF_CNT2; p.acc_init = 1; }
+    // the variants with the Philox recipe or a compensated head live in the library's second translation unit
+    if (kahan_type != 0) role_heavy_launch(round_mode, false, kahan_type, qgrid, stream, ph);
+    if (rest_tiles > 0) {
+      const bool wd = weight_decay != 0.f;
+      if (round_mode == XMC_ROUND_SR_PHILOX) role_heavy_launch(round_mode, wd, 0, qgrid, stream, p);
+      else if (round_mode == XMC_ROUND_RTN && wd) fp8_step_role_kernel<ROUND_RTN, true, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
+      else if (round_mode == XMC_ROUND_RTN) fp8_step_role_kernel<ROUND_RTN, false, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
+      else if (wd) fp8_step_role_kernel<ROUND_SR_FAST, true, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
+      else fp8_step_role_kernel<ROUND_SR_FAST, false, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
     }
-#undef XMC_LAUNCH_STEP
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;
     reduce_gx_role_kernel<<<192, 128, 0, stream>>>((const floatx4*)(ws + WS_PARTIAL), qgrid, scale_w, grad_x_f32,
                                                  (unsigned short*)grad_x_bf16, batch, (int*)(ws + WS_FLAGS), dp);
   }
   return launch_status();
+}
+
+extern "C" {
+
+int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                    int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                    float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
+                    void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream_) {
+  return fused_step(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, labels_coo, nnz, lr, seeds, round_mode,
+                    scale_w, scale_x, weight_decay, dropout_p, dropout_seed, nullptr, 0, 0, grad_x_bf16, grad_x_f32, workspace,
+                    workspace_bytes, stream_);
+}
+
+int xmc_fp8_kahan_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                       int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                       void* kahan, int kahan_type, int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                       size_t workspace_bytes, void* stream_) {
+  if (kahan_type != 1 && kahan_type != 2) return XMC_ERR_MODE;
+  return fused_step(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, labels_coo, nnz, lr, seeds, round_mode,
+                    1.0f, 1.0f, 0.0f, 0.0f, 0ull, kahan, kahan_type, num_head, grad_x_bf16, grad_x_f32, workspace,
+                    workspace_bytes, stream_);
 }
 
 int xmc_fp8_forward(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,

@@ -28,19 +28,21 @@ constexpr int MAX_WG = 256;                                   // workgroups of t
 constexpr size_t WS_XQ = 0;                                   // FP8 logits operands   BP*D
 constexpr size_t WS_XT = WS_XQ + (size_t)BP * D;              // bf16 grad_W operands  BP*D*2
 constexpr size_t WS_KEYS = WS_XT + (size_t)BP * D * 2;        // sorted positive keys  MAX_POS*4
-constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // 2048 ints: counters, XCC ids, error words (below)
-constexpr size_t WS_PARTIAL = WS_FLAGS + 8192;                // MAX_WG * 12 * 512 * 16 bytes of grad_X partials
+constexpr size_t WS_FLAGS = WS_KEYS + (size_t)MAX_POS * 4;    // 4096 ints: counters, XCC ids, error words (below)
+constexpr size_t WS_PARTIAL = WS_FLAGS + 16384;               // MAX_WG * 12 * 512 * 16 bytes of grad_X partials
 constexpr size_t WS_EXCH = WS_PARTIAL + (size_t)MAX_WG * 12 * 512 * 16;     // G exchange ring: 64 quads x 8 slots x 20 KiB
 constexpr size_t WS_TILEPTR = WS_EXCH + (size_t)(MAX_WG / 4) * 8 * 20480;   // tile_ptr[num_tiles + 1], then the tile descriptors
 
-// Layout of the 2048 ints at WS_FLAGS (all but the last cleared at the start of every step):
+// Layout of the 4096 ints at WS_FLAGS (all but the sticky word cleared at the start of every step):
 //   [0, 1024)             tiles-published counters of the persistent step kernel: sixteen per quad
+//   [QF_CNT2, +1024)      the same for the step's second launch (the head-Kahan layer runs the compensated tiles first)
 //   [QF_XCC, QF_XCC+256)  XCC id every workgroup of the step kernel found itself on
 //   [QF_ERR]              error word: bit 0 = a bounded wait expired, bit 1 = the workgroups of a quad were not placed on
 //                         one XCD (their exchange of G through that XCD's L2 is then not coherent)
 //   [QF_STICKY]           the error words of all steps since the caller last cleared it, OR-ed together by the step's
 //                         last kernel; no kernel ever clears it
-constexpr int QF_WORDS = 2048;
+constexpr int QF_WORDS = 4096;
+constexpr int QF_CNT2 = 2048;
 constexpr int QF_XCC = 1024;
 constexpr int QF_ERR = 2044;
 constexpr int QF_STICKY = 2047;

@@ -33,7 +33,8 @@ struct QuadParams {
   int num_chunks;
   int rows_per_chunk;
   int tiles_per_chunk;
-  int num_tiles;
+  int num_tiles;                      // tiles of all chunks
+  int run_tiles;                      // tiles of this launch of the step kernel (all of them, the head's or the rest)
   const unsigned char* xq;            // logits operands (layout of prep_x_quad_thread)
   const bf16x8* xt;                   // grad_W operands
   const unsigned* keys;               // sorted positives: label*256 + batch_row
@@ -41,7 +42,7 @@ struct QuadParams {
   const uint4* desc;                  // [nquads][kmax][2] tile descriptors written by quad_desc_prep_kernel: the tiles of
                                       // one quad are consecutive entries, in the order the quad walks them
   int nquads;                         // quads of the step kernel's launch (grid / 4)
-  int kmax;                           // descriptor entries per quad = ceil(num_tiles / nquads)
+  int kmax;                           // descriptor entries per quad = ceil(run_tiles / nquads)
   floatx4* partial;                   // [gridDim.x][24][256] per-workgroup grad_X partial sums
   unsigned char* exch;                // [nquads][QSLOTS][QG_BYTES] G exchange ring
   int* flags;                         // [nquads][16] tiles-published counters; [QF_XCC + g] XCC ids; [QF_ERR] error word
@@ -49,6 +50,13 @@ struct QuadParams {
   float lr_eff;                       // lr / scale_w
   float wd_eff;                       // weight decay x scale_w (applied to the codes)
   int batch;
+  // Head-Kahan layer (chunked_head_kahan_fp8xmc_clf.py:127-131): the first num_head rows of chunk 0 carry a compensation
+  // term.  The tiles that contain such rows (the first head_tiles of chunk 0) are a launch of their own, with their own
+  // descriptor table (kmax_head entries per quad, in front of the table of the other tiles) and counters.
+  unsigned char* kahan;               // [num_head, 768] bf16 or e5m2, or null
+  int num_head, head_tiles, kmax_head;
+  int cnt_base;                       // first of this launch's tiles-published counters in flags
+  int acc_init;                       // the grad_X partials continue from what the launch before left in `partial`
 };
 
 #define QFENCE() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point
@@ -120,6 +128,7 @@ __device__ __forceinline__ QTile q_desc_full(q_cdesc* desc, int t) {
   return q;
 }
 
+#ifndef XMC_HEAVY_TU   // the kernels below are compiled once, in the library's main translation unit
 // First of the two launches in front of the step kernel: clear the counters (flags, may be null) and sort the positives
 // (key = label*256 + (batch row - row0) for the batch rows row0..row0+255 that lie below `batch`; every other entry, and
 // labels outside the label space, -> 0xFFFFFFFF) by rank.  Workgroup b ranks keys 64b..64b+63 of the n_pad
@@ -131,7 +140,8 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
   extern __shared__ unsigned sk[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   if (blockIdx.x == 0 && flags)
-    for (int i = tid; i < QF_STICKY; i += 256) flags[i] = 0;
+    for (int i = tid; i < QF_WORDS; i += 256)
+      if (i != QF_STICKY) flags[i] = 0;
   if (n_pad == 0) return;
   // eight (row, label) pairs per thread in flight at a time: the loads miss every cache
   const int2* coo2 = (const int2*)coo;
@@ -236,9 +246,15 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
     const unsigned long long base = (unsigned long long)(p.chunk[c] + (size_t)row0 * D);
     // tile t is position t / nquads of quad t % nquads: a quad reads its descriptors as one contiguous run, so the
     // scalar cache serves all but one fetch in two
-    const int slot = (t % p.nquads) * p.kmax + t / p.nquads;
+    // With a compensated head its tiles have a table of their own in front; behind the head the row a tile records
+    // counts from the head's end (the reference updates those rows through sliced tensors, so the offsets of its random
+    // numbers restart there: chunked_head_kahan_fp8xmc_clf.py:130-131).
+    const bool behind = t >= p.head_tiles;
+    const int tl = behind ? t - p.head_tiles : t, km = behind ? p.kmax : p.kmax_head;
+    const int slot = (behind ? p.nquads * p.kmax_head : 0) + (tl % p.nquads) * km + tl / p.nquads;
+    const int row_rec = row0 - (behind && c == 0 ? p.num_head : 0);
     desc[2 * slot] = uint4{(unsigned)base, (unsigned)(base >> 32), (unsigned)min(TL, p.rows_per_chunk - row0), p.seed[c]};
-    desc[2 * slot + 1] = uint4{(unsigned)p0, (unsigned)p1, (unsigned)row0, (unsigned)(c * p.rows_per_chunk + row0)};
+    desc[2 * slot + 1] = uint4{(unsigned)p0, (unsigned)p1, (unsigned)row_rec, (unsigned)(c * p.rows_per_chunk + row0)};
   }
 }
 
@@ -281,5 +297,7 @@ __device__ __forceinline__ void prep_x_quad_thread(int i, const unsigned short* 
     xt[off] = raw[q];
   }
 }
+
+#endif  // XMC_HEAVY_TU
 
 }  // namespace xmc

@@ -39,6 +39,11 @@ constexpr int RC_RING = RQ + 1;             // own-column images: in use, RQ - 1
 #define XMC_PD 3
 #endif
 constexpr int NB_B = XMC_NB_B;              // A^T blocks (16 label rows) of a tile the B wavefronts take; the A wavefronts take the rest
+// with a compensated head (KT != 0) the B wavefronts take all four: they alone then touch the compensation buffer, with
+// ordinary loads and stores whose completion the compiler tracks (the A wavefronts count their loads by hand)
+// With the reference's Philox recipe the update is a hundred vector instructions per weight and bounds the kernel: the
+// two wavefronts of a SIMD then share it evenly.
+constexpr int r_nbb(int kt, int mode) { return kt != 0 ? 4 : mode == ROUND_SR_PHILOX ? 2 : NB_B; }
 constexpr int RR_RING = 3;                  // own-rows images: in use, landed, landing
 constexpr int RG_BUF = 2;                   // gathered G tiles: in use, landing
 constexpr int RG_BYTES = 16384;             // one G tile: 4 members x 128 rows x 32 bytes
@@ -51,7 +56,7 @@ constexpr int RLDS_G = RLDS_O + RO_RING * RO_BYTES;
 constexpr int RLDS_R = RLDS_G + RG_BUF * RG_BYTES;
 constexpr int RLDS_M = RLDS_R + RR_RING * RROW_BYTES;   // per A wavefront two snapshots of four counters (32 bytes); at +128 two abort words
 constexpr int RLDS_BYTES = RLDS_M + 256;
-constexpr int RF_CNT = 0;                   // flags[RF_CNT + quad*16 + member*4 + A wavefront]: tiles published
+// tiles-published counters: flags[p.cnt_base + quad*16 + member*4 + A wavefront]
 
 static_assert(RLDS_BYTES <= 160 * 1024, "LDS budget");
 
@@ -83,13 +88,37 @@ struct RBlockLane {
   unsigned char* dummy;  // where stores of rows past the end of a chunk go (nobody reads it)
 };
 
+// The compensation terms of one A^T block (head-Kahan layer): 12 per lane, raw (bf16: six dwords, e5m2: three), and
+// whether the lane's row carries one at all.
+struct RKahanBlock { unsigned raw[6]; bool head; int row; };
+
 // piece c (0..7) of the update of A^T block nb (12 weights per lane): pieces 0-2 decode the old weights and form
 // T = W - lr A, 3-5 make the random words' hashes, 6-7 round, 7 stores.  Split so that the vector instructions can be
 // issued between matrix instructions.  With MODE.FP16_OVFL set the fp8 converters saturate, so nothing is clamped here.
-template <int MODE, bool WD>
+//
+// KT != 0 (compensation buffer of bf16 (1) or e5m2 (2) values, chunked_head_kahan_fp8xmc_clf.py:127-131 with
+// fuse_kernel.py:237-262): on rows that carry a term k the update is
+//   T = (W + k) - lr A,  W' = round(T),  k' = cast(((k + W) - W') - lr A)
+// and on the other rows of the tile (behind the head's end) the plain update, whose random offsets count from that end.
+template <int MODE, bool WD, int KT>
 __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab)[3], const unsigned (&wq)[3], float (&t)[3][4],
                                                unsigned (&hs)[3], unsigned (&outw)[3], const RBlockLane& bl, const QTile& q,
-                                               unsigned hash_tile, float lr_eff, float wd_eff, int l16, qlds_u8* lds, unsigned oimg) {
+                                               unsigned hash_tile, float lr_eff, float wd_eff, int l16, qlds_u8* lds, unsigned oimg,
+                                               const RKahanBlock& kb, unsigned char* kahan, int num_head) {
+  // W + k of column group cg (exact decode of both; k = 0 on rows without a term)
+  auto kahan_sum = [&](int cg, float (&s)[4]) {
+    const unsigned wv = wq[cg];
+    floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, true);
+    float k[4];
+    if (KT == 1) {
+      k[0] = __uint_as_float(kb.raw[2 * cg] << 16); k[1] = __uint_as_float(kb.raw[2 * cg] & 0xFFFF0000u);
+      k[2] = __uint_as_float(kb.raw[2 * cg + 1] << 16); k[3] = __uint_as_float(kb.raw[2 * cg + 1] & 0xFFFF0000u);
+    } else {
+      floatx2 k01 = __builtin_amdgcn_cvt_pk_f32_bf8((int)kb.raw[cg], false), k23 = __builtin_amdgcn_cvt_pk_f32_bf8((int)kb.raw[cg], true);
+      k[0] = k01.x; k[1] = k01.y; k[2] = k23.x; k[3] = k23.y;
+    }
+    s[0] = w01.x + k[0]; s[1] = w01.y + k[1]; s[2] = w23.x + k[2]; s[3] = w23.y + k[3];
+  };
 #ifdef XMC_X_NOUPDATE
   if (c == 7 && ab[0][0] + ab[1][1] + ab[2][2] == 1.2345f) *(volatile unsigned*)bl.dummy = wq[0] + wq[1] + wq[2];
   return;
@@ -98,7 +127,12 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
     const int cg = c;
     const unsigned wv = wq[cg];
     floatx2 w01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, false), w23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv, true);
-    if (WD) {   // T = W - lr (A + wd W): the decayed gradient first, in fp32
+    if (KT != 0) {
+      float s[4];
+      kahan_sum(cg, s);
+#pragma unroll
+      for (int e = 0; e < 4; e++) t[cg][e] = __builtin_fmaf(-lr_eff, ab[cg][e], s[e]);
+    } else if (WD) {   // T = W - lr (A + wd W): the decayed gradient first, in fp32
       t[cg][0] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w01.x, ab[cg][0]), w01.x);
       t[cg][1] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w01.y, ab[cg][1]), w01.y);
       t[cg][2] = __builtin_fmaf(-lr_eff, __builtin_fmaf(wd_eff, w23.x, ab[cg][2]), w23.x);
@@ -116,8 +150,22 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
       h ^= h >> 16; h *= 0x85EBCA77u; h ^= h >> 15;
       hs[cg] = h;
     }
+    if (MODE == ROUND_SR_PHILOX) {
+      // the reference's recipe on this column group's four targets, one Philox word after the other: the counter of
+      // the next word passes through an opaque statement together with this word's result, so that the four chains of
+      // ten rounds are not interleaved (forty live registers that this kernel does not have)
+      const int row = 16 * nb + l16;
+      const int rrow = KT != 0 ? (kb.head ? kb.row : kb.row - num_head) : q.row0 + row;
+      unsigned off = (unsigned)rrow * (unsigned)D + bl.gcol + 4 * cg;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const unsigned r = philox_word0(off + e, q.seed, 0u) & 0xFFFFFu;
+        unsigned tb = (__float_as_uint(t[cg][e]) + r) & 0xFFF00000u;
+        asm volatile("" : "+v"(off), "+v"(tb));
+        t[cg][e] = __uint_as_float(tb);
+      }
+    }
   } else {
-    const int row = 16 * nb + l16;
 #pragma unroll
     for (int cg = (c == 6 ? 0 : 2); cg < (c == 6 ? 2 : 3); cg++) {
       if (MODE == ROUND_SR_FAST) {
@@ -129,7 +177,32 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
         packed = __builtin_amdgcn_cvt_sr_fp8_f32(t[cg][3], fast_word(hs[cg], 3), packed, 3);
         outw[cg] = (unsigned)packed;
       } else {
-        outw[cg] = round4<MODE>(t[cg][0], t[cg][1], t[cg][2], t[cg][3], (unsigned)(q.row0 + row), q.label0 + (unsigned)row, bl.gcol + 4 * cg, q.seed);
+        // round to nearest (the Philox recipe has been applied to T by now); the converter saturates
+        int packed;
+        asm volatile("" : "=v"(packed));   // every byte is written below
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[cg][0], t[cg][1], packed, false);
+        packed = __builtin_amdgcn_cvt_pk_fp8_f32(t[cg][2], t[cg][3], packed, true);
+        outw[cg] = (unsigned)packed;
+      }
+      if (KT != 0) {
+        float s[4], kn[4];
+        kahan_sum(cg, s);
+        floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)outw[cg], false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)outw[cg], true);
+        kn[0] = __builtin_fmaf(-lr_eff, ab[cg][0], s[0] - n01.x); kn[1] = __builtin_fmaf(-lr_eff, ab[cg][1], s[1] - n01.y);
+        kn[2] = __builtin_fmaf(-lr_eff, ab[cg][2], s[2] - n23.x); kn[3] = __builtin_fmaf(-lr_eff, ab[cg][3], s[3] - n23.y);
+        // this column group's new terms straight to memory (8 or 4 bytes per lane; the buffer is touched once per step)
+        if (kb.head) {
+          if (KT == 1) {
+            *(uint2*)(kahan + ((size_t)kb.row * D + bl.gcol + 4 * cg) * 2) = uint2{bf16_pack2(kn[0], kn[1]), bf16_pack2(kn[2], kn[3])};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
+            int pk = 0;
+            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
+            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
+            *(unsigned*)(kahan + (size_t)kb.row * D + bl.gcol + 4 * cg) = (unsigned)pk;
+          }
+        }
       }
     }
     if (c == 7) {
@@ -145,8 +218,10 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
   }
 }
 
-template <int MODE, bool WD>
+template <int MODE, bool WD, int KT>
 __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams p) {
+  constexpr int NBB = r_nbb(KT, MODE);          // A^T blocks of a tile the B wavefronts take
+  constexpr int NBA = 4 - NBB > 0 ? 4 - NBB : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   qlds_u8* lds = (qlds_u8*)lds_raw;
   // fp8 conversions saturate at +-448 instead of returning NaN (MODE.FP16_OVFL; infinities and NaN still give NaN)
@@ -158,7 +233,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   const int xcd = g & 7, j = g >> 3, m = j & 3;
   const int nquads = gridDim.x >> 2;
   const int quad = (j >> 2) * 8 + xcd;
-  const int n_it = quad < p.num_tiles ? (p.num_tiles - quad + nquads - 1) / nquads : 0;
+  const int n_it = quad < p.run_tiles ? (p.run_tiles - quad + nquads - 1) / nquads : 0;
 
   q_cdesc* cdesc = (q_cdesc*)p.desc;
   // descriptor entry of position k in this quad's sequence; positions past the end fall back to entry 0 (tile 0), whose
@@ -200,8 +275,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   if (v < 4) {
     // =========================================================================================== A wavefronts
     const int a = v;
-    int* myflag = p.flags + RF_CNT + quad * 16 + m * 4 + a;
-    const int* srcflags = p.flags + RF_CNT + quad * 16 + a * 4;
+    int* myflag = p.flags + p.cnt_base + quad * 16 + m * 4 + a;
+    const int* srcflags = p.flags + p.cnt_base + quad * 16 + a * 4;
     const __attribute__((address_space(4))) unsigned* ckeys = (const __attribute__((address_space(4))) unsigned*)p.keys;
 
     intx8 xq[2][6];   // logits operands: batch blocks 2a, 2a+1, K steps of 128
@@ -467,20 +542,20 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       const unsigned gb = (unsigned)(RLDS_G + (i & 1) * RG_BYTES);
       const unsigned gwl = gb + bl.bg_lane, gwh = gb + (bl.bg_lane ^ 128u), wrow = wc + bl.wrow_lane;
       const unsigned oimg = (unsigned)(RLDS_O + (i & 1) * RO_BYTES);
-      floatx4 aa[4 - NB_B][3];
-      unsigned wq[4 - NB_B][3];
+      floatx4 aa[NBA][3];
+      unsigned wq[NBA][3];
 #pragma unroll
-      for (int nb = NB_B; nb < 4; nb++) {
+      for (int nb = NBB; nb < 4; nb++) {
         bf16x8 bg[4];
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) bg[ks] = read_bg(gwl, gwh, nb, ks);
 #pragma unroll
-        for (int cg = 0; cg < 3; cg++) wq[nb - NB_B][cg] = *(const unsigned*)(lds + wrow + 16 * nb * QWS + 4 * cg);
+        for (int cg = 0; cg < 3; cg++) wq[nb - NBB][cg] = *(const unsigned*)(lds + wrow + 16 * nb * QWS + 4 * cg);
 #pragma unroll
         for (int ks = 0; ks < 4; ks++)
 #pragma unroll
           for (int cg = 0; cg < 3; cg++)
-            aa[nb - NB_B][cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][ks], bg[ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : aa[nb - NB_B][cg], 0, 0, 0);
+            aa[nb - NBB][cg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xt[cg][ks], bg[ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : aa[nb - NBB][cg], 0, 0, 0);
         QFENCE();
       }
       // descriptors of the next iteration: requested here, in front of a long stretch of vector work, because every wait
@@ -500,18 +575,19 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       {
         float t[3][4];
         unsigned hs[3], outw[3];
+        const RKahanBlock nok = {};
         const unsigned hash_tile = qb.label0 * (unsigned)(D / 4) * 0x9E3779B1u + qb.seed;
         const int rslot = sa == 0 ? RR_RING - 1 : sa - 1;   // (i + RQ + RR_RING - 1) % RR_RING
 #pragma unroll
-        for (int nb = NB_B; nb < 4; nb++)
+        for (int nb = NBB; nb < 4; nb++)
 #pragma unroll
           for (int c = 0; c < 8; c++) {
-            constexpr int every = 2 * (4 - NB_B);
-            const int pc = (nb - NB_B) * 8 + c;
+            constexpr int every = 2 * NBA;
+            const int pc = (nb - NBB) * 8 + c;
             if (pc % every == 0) rows_piece(rslot, qr, pc / every);
-            r_update_piece<MODE, WD>(c, nb, aa[nb - NB_B], wq[nb - NB_B], t, hs, outw, bl, qb, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
+            r_update_piece<MODE, WD, 0>(c, nb, aa[nb - NBB], wq[nb - NBB], t, hs, outw, bl, qb, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, nok, nullptr, 0);
           }
-        if (NB_B == 4) rows_pieces(rslot, qr);
+        if (NBB == 4) rows_pieces(rslot, qr);
       }
       RT_NOW(rt_t1); RT_ADD(5, rt_t0, rt_t1);
       // Loads and stores complete in order.  Waiting for all but the stores of G and the rows covers the gather, the
@@ -544,10 +620,15 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   __builtin_amdgcn_s_setprio(3);
 #endif
   floatx4 acc2[8][3];    // grad_X[128 batch rows x 48 features]
+  {
+    // a second launch of a step continues the sums of the first
+    const floatx4* prev = p.partial + (size_t)g * 24 * 256;
 #pragma unroll
-  for (int mb = 0; mb < 8; mb++)
+    for (int mb = 0; mb < 8; mb++)
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) acc2[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int nn = 0; nn < 3; nn++)
+        acc2[mb][nn] = p.acc_init ? prev[(mb * 3 + nn) * 256 + s * 64 + lane] : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   // per-lane parts of the LDS addresses
   const unsigned ga_lane = (unsigned)((kg >> 1) * 4096 + g_row16(l16) * 32 + ((kg & 1) ^ (l16 >> 3)) * 16);           // grad_X operand
@@ -614,15 +695,15 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     const unsigned wtr = wc + wtr_lane, wrow = wc + bl.wrow_lane;
     const unsigned hash_tile = q.label0 * (unsigned)(D / 4) * 0x9E3779B1u + q.seed;
 
-    // The tile is a sequence of 16 + 4 NB_B steps of one LDS operand and three matrix instructions each.  The first
-    // 8 NB_B alternate:
+    // The tile is a sequence of 16 + 4 NBB steps of one LDS operand and three matrix instructions each.  The first
+    // 8 NBB alternate:
     //   even step 8o + 2ks:      A^T block o (label rows 16o..), K step ks:  aa[cg] += X^T[cg][ks] * G^T   (operand: two transposing reads)
     //   odd  step 8o + 2j + 1:   grad_X step 4o + j
     // and the rest are the remaining grad_X steps; grad_X step x = K step x/8 (32 labels), batch block x%8:
     //   acc2[mb][nn] += G^T * W[nn]  (operand: one 16-byte read).
     // The operand of step k + 3 is requested in step k.  The vector work of the update of block o (12 weights per lane,
     // eight pieces) is spread over the steps behind the block's last, so that it issues between the matrix instructions.
-    constexpr int NS = 16 + 4 * NB_B, NALT = 8 * NB_B;
+    constexpr int NS = 16 + 4 * NBB, NALT = 8 * NBB;
     constexpr int PD = XMC_PD;   // operands are requested this many steps ahead
     bf16x8 op[NS + PD];
     auto request = [&](int k) {
@@ -653,6 +734,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     float t[3][4];
     unsigned hs[3], outw[3];
     intx4 so_v;   // a piece of the previous tile's updated weights on its way from LDS to memory
+    RKahanBlock kb[2] = {};   // compensation terms of the block in progress and of the one being rounded
+    // (this loop must be unrolled completely: its register arrays are indexed by k.  The variants with the Philox
+    // recipe or a compensated head exceed the compiler's default size limit for "#pragma unroll" and are compiled in a
+    // translation unit of their own, xmc_fp8_role_heavy.hip, with a higher limit.)
 #pragma unroll
     for (int k = 0; k < NS; k++) {
       if ((k & 7) == 1 && k < 24) so_v = so_read((i + 1) & 1, k >> 3);
@@ -676,15 +761,36 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 #pragma unroll
         for (int cg = 0; cg < 3; cg++) wq[o & 1][cg] = *(const unsigned*)(lds + wrow + 16 * o * QWS + 4 * cg);
       }
+      if (KT != 0 && k < NALT && (k & 7) == 0) {
+        const int o = k >> 3;
+        {
+          // the block's compensation terms: 24 (bf16) or 12 (e5m2) bytes per lane, from memory to registers; rows
+          // behind the head's end (or the chunk's) read row 0 and count as zero
+          RKahanBlock& kk = kb[o & 1];
+          kk.row = q.row0 + 16 * o + l16;
+          kk.head = kk.row < p.num_head;
+          const unsigned char* src = p.kahan + ((size_t)(kk.head ? kk.row : 0) * D + bl.gcol) * (KT == 1 ? 2 : 1);
+          if (KT == 1) {
+#pragma unroll
+            for (int cg = 0; cg < 3; cg++) {
+              const uint2 kv = *(const uint2*)(src + 8 * cg);
+              kk.raw[2 * cg] = kk.head ? kv.x : 0u; kk.raw[2 * cg + 1] = kk.head ? kv.y : 0u;
+            }
+          } else {
+#pragma unroll
+            for (int cg = 0; cg < 3; cg++) { const unsigned kv = *(const unsigned*)(src + 4 * cg); kk.raw[cg] = kk.head ? kv : 0u; }
+          }
+        }
+      }
       if (k >= 8 && k < NALT) {
         const int o = (k >> 3) - 1;
-        r_update_piece<MODE, WD>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
-      } else if (k >= NALT && NB_B > 0) {
-        constexpr int per = NB_B == 4 ? 8 : 8 / (16 - 4 * NB_B);   // pieces per trailing step
-        const int o = NB_B - 1;
+        r_update_piece<MODE, WD, KT>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
+      } else if (k >= NALT && NBB > 0) {
+        constexpr int per = NBB == 4 ? 8 : 8 / (16 - 4 * NBB);   // pieces per trailing step
+        const int o = NBB - 1;
 #pragma unroll
         for (int c = (k - NALT) * per; c < (k - NALT + 1) * per && c < 8; c++)
-          r_update_piece<MODE, WD>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
+          r_update_piece<MODE, WD, KT>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
       }
       if (k < NALT && (k & 1) == 0) {
         const int o = k >> 3, ks = (k & 7) >> 1;
@@ -701,9 +807,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       QFENCE();
 #endif
     }
-    if (NB_B == 4) {
+    if (NBB == 4) {
 #pragma unroll
-      for (int c = 0; c < 8; c++) r_update_piece<MODE, WD>(c, 3, aa[1], wq[1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg);
+      for (int c = 0; c < 8; c++) r_update_piece<MODE, WD, KT>(c, 3, aa[1], wq[1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[1], p.kahan, p.num_head);
     }
     q_p = q;
     q_n = q_desc_full(cdesc, tile_at(i + 1));
@@ -726,6 +832,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + s * 64 + lane] = acc2[mb][nn];
 }
 
+#ifndef XMC_HEAVY_TU
 // grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768].  192 workgroups of 128
 // threads: workgroup (block, m, part) covers lanes 128 part.. of the 256 B-wavefront lanes of a step workgroup.
 __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
@@ -766,5 +873,12 @@ __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* part
     }
   }
 }
+
+#endif  // XMC_HEAVY_TU
+
+// The variants of fp8_step_role_kernel with the reference's Philox recipe (XMC_ROUND_SR_PHILOX) or a compensated head
+// (kahan_type 1, 2), defined in xmc_fp8_role_heavy.hip: opt in to the LDS size (once per device); launch.
+void role_heavy_set_lds();
+void role_heavy_launch(int round_mode, bool weight_decay, int kahan_type, int grid, hipStream_t stream, const QuadParams& p);
 
 }  // namespace xmc

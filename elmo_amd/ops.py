@@ -76,6 +76,37 @@ def fp8_step(chunks, x, labels, lr, seeds=None, round_mode="rtn", scale_w=1.0, s
     return (grad_out, gf) if want_f32 else grad_out
 
 
+def fp8_kahan_step(chunks, kahan, num_head, x, labels, lr, seeds=None, round_mode="rtn", workspace=None, grad_out=None,
+                   want_f32=False):
+    """One fused step of the head-Kahan layer (reference: chunked_head_kahan_fp8xmc_clf.py:95-133): as fp8_step, and the
+    first num_head rows of chunk 0 are updated with the compensation buffer `kahan` ([num_head, 768] bf16 or
+    float8_e5m2, updated in place)."""
+    lib = _lib.load()
+    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2
+    assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
+    assert labels.dim() == 2 and labels.shape[1] == 2
+    batch, feat = x.shape
+    arr, rows = _chunk_array(chunks)
+    nc = len(chunks)
+    assert kahan.is_cuda and kahan.is_contiguous() and kahan.shape == (num_head, FEATURES)
+    assert kahan.dtype in (torch.bfloat16, torch.float8_e5m2) and 0 < num_head <= rows
+    if workspace is None:
+        workspace = alloc_workspace(nc, rows, x.device)
+    if grad_out is None:
+        grad_out = torch.empty(batch, feat, dtype=torch.bfloat16, device=x.device)
+    gf = torch.empty(batch, feat, dtype=torch.float32, device=x.device) if want_f32 else None
+    sarr = None
+    if seeds is not None:
+        sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
+    st = lib.xmc_fp8_kahan_step(arr, nc, rows, x.data_ptr(), batch, feat, labels.data_ptr() if labels.numel() else None,
+                                labels.shape[0], float(lr), sarr, _lib.ROUND_MODES[round_mode], kahan.data_ptr(),
+                                1 if kahan.dtype == torch.bfloat16 else 2, int(num_head), grad_out.data_ptr(),
+                                gf.data_ptr() if gf is not None else None, workspace.data_ptr(), workspace.numel(),
+                                _stream_ptr())
+    _lib.check(st, "xmc_fp8_kahan_step")
+    return (grad_out, gf) if want_f32 else grad_out
+
+
 def fp8_forward(chunks, x, num_labels, scale_w=1.0, scale_x=1.0, workspace=None):
     """Inference logits [B, num_labels] bf16 (reference: chunked_fp8xmc_clf.py:45-60).  Any batch size: rows are
     processed in slices of at most 128, the last one padded to a multiple of 16."""

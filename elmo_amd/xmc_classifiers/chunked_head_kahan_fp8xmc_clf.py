@@ -6,12 +6,13 @@ bf16 or float8_e5m2, `num_head`, `grad_input`, `_dtype`, `iteration`) and config
 (training.FP8.using_head_kahan, training.FP8.fp8_head_kahan, training.FP8.head_ratio, training.xmc.simulated_fp8).
 
 Without the compensation buffer (using_head_kahan false) and without simulated FP8 the step is the fused kernel of
-Fp8XMCBCEChunkedLayer.  With the buffer the step runs on the three-kernel path in true-FP8 arithmetic (logits from
-e4m3(X), saturating cast), whose update kernel carries the Kahan recurrence of fuse_kernel.py:202-262 for the first
-num_head rows of chunk 0.  As in the reference, simulated FP8 takes precedence over the compensation (:122-124).
+Fp8XMCBCEChunkedLayer.  With the buffer the step is the fused kernel as well (ops.fp8_kahan_step: the tiles that hold
+head rows run first, in a variant of the kernel that carries the Kahan recurrence of fuse_kernel.py:202-262 for the
+first num_head rows of chunk 0; the other tiles follow in the plain kernel) whenever the batch is a multiple of 16;
+any other batch runs on the three-kernel path in the same true-FP8 arithmetic (logits from e4m3(X), saturating cast).
+As in the reference, simulated FP8 takes precedence over the compensation (:122-124).
 
-Optional, not in the reference: training.xmc.rounding ("sr_philox" default with the buffer or simulated FP8, else
-"sr_fast"; "rtn").
+Optional, not in the reference: training.xmc.rounding ("sr_philox" default with simulated FP8, else "sr_fast"; "rtn").
 """
 import torch
 from torch import nn
@@ -63,8 +64,8 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
             self.head_kahan = torch.zeros(self.num_head, features, dtype=kdt, device=self.device)
             assert 0 < self.num_head <= self.num_labels_i
         self._tiled = bool(self.fake_fp8_matmul or self.using_head_kahan)
-        self.rounding = _opt(cfg.training.xmc, "rounding", "sr_philox" if self._tiled else "sr_fast")
-        assert self.rounding in (("sr_philox", "rtn") if self._tiled else ("sr_fast", "sr_philox", "rtn"))
+        self.rounding = _opt(cfg.training.xmc, "rounding", "sr_philox" if self.fake_fp8_matmul else "sr_fast")
+        assert self.rounding in (("sr_philox", "rtn") if self.fake_fp8_matmul else ("sr_fast", "sr_philox", "rtn"))
         self.block_size = 16
         self.loss = torch.tensor(0.0, device=self.device)
         self.iteration = 0
@@ -116,6 +117,9 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace)
+        elif self.using_head_kahan and embed.shape[0] % 16 == 0:
+            self.grad_input = ops.fp8_kahan_step(self._chunks(), self.head_kahan, self.num_head, x, lab, xmc_lr[0],
+                                                 seeds=seeds, round_mode=self.rounding, workspace=self._workspace)
         elif self.using_head_kahan:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,

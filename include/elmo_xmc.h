@@ -93,6 +93,21 @@ int xmc_fp8_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk,
                     float scale_w, float scale_x, float weight_decay, float dropout_p, unsigned long long dropout_seed,
                     void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The fused step of the head-Kahan layer (src/xmc_classifiers/chunked_head_kahan_fp8xmc_clf.py:95-133, update of the
+ * head rows: :127-129 with src/triton_kernels/fuse_kernel.py:202-262): as xmc_fp8_step with scales 1, and the first
+ * num_head rows of chunk 0 carry a compensation term,
+ *     T = (W + k) - lr A,   W' = round(T),   k' = cast(((k + W) - W') - lr A).
+ * The rows of chunk 0 behind the head are updated as the reference updates them, through tensors sliced at num_head
+ * (:130-131): the offsets of XMC_ROUND_SR_PHILOX's random numbers count from there.
+ *   kahan        device [num_head, 768], updated in place: bf16 (kahan_type 1) or float8_e5m2 (kahan_type 2, saturating
+ *                cast), 16-byte aligned
+ *   num_head     1 .. rows_per_chunk
+ * The tiles that hold head rows run as a launch of their own in front of the other tiles' launch.  Same status codes. */
+int xmc_fp8_kahan_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, const void* x_bf16, int batch,
+                       int features, const int32_t* labels_coo, int nnz, float lr, const uint32_t* seeds, int round_mode,
+                       void* kahan, int kahan_type, int num_head, void* grad_x_bf16, float* grad_x_f32, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* Inference logits (chunked_fp8xmc_clf.py:45-60): out[b, label] = bf16(scale * sum_k e4m3(X/scale_x)[b,k] * W[label,k])
  * for label < num_labels (the padding rows of the last chunk are dropped, :60).
  *   out_bf16        device [batch, out_stride] bf16, out_stride >= num_labels; any alignment works, rows that start

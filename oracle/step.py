@@ -119,7 +119,8 @@ def fp8_step(w_codes, x_bf16, labels, lr, *, seeds=None, sr_mode="rtn", simulate
     return out + (parts,) if return_parts else out
 
 
-def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="bf16", seeds=None, sr_mode="rtn"):
+def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="bf16", seeds=None, sr_mode="rtn",
+                   rand_fn=None):
     """One step of the head-Kahan FP8 layer (chunked_head_kahan_fp8xmc_clf.py:95-133; fuse_kernel.py:202-262), true FP8.
 
     Logits, G and grad_X exactly as fp8_step.  Update of chunk 0 (:127-131): rows [0, num_head) carry a compensation
@@ -129,6 +130,8 @@ def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="
         k' = cast( ((f32(k) + f32(W)) - f32(Wq)) - lr*A )
     with random offsets row*d + col; the remaining rows of chunk 0 are updated by a call on the sliced tensors, so
     their offsets restart at zero: (row - num_head)*d + col.  Other chunks as in fp8_step.
+    sr_mode "exact" (this build's fast mode, not in the reference): exact stochastic rounding on the e4m3 grid with the
+    words rand_fn(chunk, row_in_chunk * d + col), rows counted from the chunk's start everywhere.
     Returns (new_codes list, new_kahan, gx_fp32, grad_input)."""
     x = np.ascontiguousarray(x_bf16, dtype=np.float32)
     B, d = x.shape
@@ -141,9 +144,11 @@ def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="
     k_old = (C.e5m2_decode(kahan) if kahan_type == "e5m2" else np.asarray(kahan, dtype=np.float32)).astype(np.float32)
     new_codes, new_kahan = [], None
 
-    def rnd(t, seed, offs):
+    def rnd(t, seed, offs, c=0, row0=0):
         if sr_mode == "rtn":
             return C.e4m3_encode(t, saturate=True)
+        if sr_mode == "exact":
+            return C.sr_e4m3_exact(t, rand_fn(c, offs + row0 * d))
         return C.e4m3_encode(C.sr_add_mask(t, C.tl_randint(seed, offs), 20), saturate=True)
 
     for c in range(nc):
@@ -164,14 +169,14 @@ def fp8_kahan_step(w_codes, kahan, x_bf16, labels, lr, num_head, *, kahan_type="
             s = (wh + k_old).astype(np.float32)                                     # weights + kahan
             t = (s.astype(np.float64) - lr64 * ah).astype(np.float32)               # - lr*acc
             offs = np.arange(num_head, dtype=np.int64)[:, None] * d + cols
-            codes[:num_head] = rnd(t, seed, offs)
+            codes[:num_head] = rnd(t, seed, offs, c, 0)
             wq = C.e4m3_decode(codes[:num_head])
             u = ((k_old + wh).astype(np.float32) - wq).astype(np.float32)           # kahan + old - new
             kn = (u.astype(np.float64) - lr64 * ah).astype(np.float32)              # - lr*acc
             new_kahan = C.e5m2_encode(kn, saturate=True) if kahan_type == "e5m2" else C.bf16_round(kn)
         t = (w64[lo:] - lr64 * a[lo:].astype(np.float64)).astype(np.float32)
         offs = np.arange(Lc - lo, dtype=np.int64)[:, None] * d + cols
-        codes[lo:] = rnd(t, seed, offs)
+        codes[lo:] = rnd(t, seed, offs, c, lo)
         new_codes.append(codes)
     gx32 = gx.astype(np.float32)
     return new_codes, new_kahan, gx32, C.bf16_round(gx32)

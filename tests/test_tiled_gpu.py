@@ -294,7 +294,7 @@ def test_fp8_module_simulated_mode(gpu):
     assert xfc.grad_input.shape == (32, 768)
 
 
-def run_kahan(case, k0, ktype, nh, device, mode, seeds, lr=0.05):
+def run_kahan(case, k0, ktype, nh, device, mode, seeds, lr=0.05, path="tiled"):
     import torch
     from elmo_amd import ops
     chunks, x, labels = H.to_device_case(case, device)
@@ -302,26 +302,42 @@ def run_kahan(case, k0, ktype, nh, device, mode, seeds, lr=0.05):
         kt = torch.from_numpy(k0.copy()).to(device).view(torch.float8_e5m2)
     else:
         kt = torch.from_numpy(C.bf16_bits(k0).view(np.int16)).to(device).view(torch.bfloat16)
-    g, gf = ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", x, labels, lr, seeds=seeds, round_mode=mode, want_f32=True,
-                           quantize_x=True, saturate=True, kahan=kt, num_head=nh)
+    if path == "fused":
+        ws = ops.alloc_workspace(len(chunks), chunks[0].shape[0], device)
+        g, gf = ops.fp8_kahan_step(chunks, kt, nh, x, labels, lr, seeds=seeds, round_mode=mode, want_f32=True, workspace=ws)
+        assert ops.step_error_word(ws, len(chunks), chunks[0].shape[0]) == 0
+    else:
+        g, gf = ops.tiled_step(chunks, chunks[0].shape[0], "e4m3", x, labels, lr, seeds=seeds, round_mode=mode, want_f32=True,
+                               quantize_x=True, saturate=True, kahan=kt, num_head=nh)
     kn = kt.view(torch.uint8).cpu().numpy() if ktype == "e5m2" else kt.float().cpu().numpy()
     return H.chunks_to_numpy(chunks), kn, gf.cpu().numpy(), g.float().cpu().numpy()
 
 
-@pytest.mark.parametrize("ktype,mode", [("bf16", "rtn"), ("bf16", "sr_philox"), ("e5m2", "rtn")])
-def test_head_kahan_parity(gpu, ktype, mode):
-    """True-FP8 arithmetic on the three-kernel path with the compensated head (fuse_kernel.py:202-262)."""
-    case = H.make_case(2, 512, 32, 81)
-    nh = 208
+@pytest.mark.parametrize("path,shape", [("tiled", (2, 512, 32, 208)), ("fused", (2, 512, 32, 208)),
+                                        ("fused", (3, 8192, 128, 8192)), ("fused", (1, 4096, 48, 4001))])
+@pytest.mark.parametrize("ktype,mode", [("bf16", "rtn"), ("bf16", "sr_philox"), ("e5m2", "rtn"), ("bf16", "sr_fast"),
+                                        ("e5m2", "sr_fast")])
+def test_head_kahan_parity(gpu, ktype, mode, path, shape):
+    """True-FP8 arithmetic with the compensated head (fuse_kernel.py:202-262) on the three-kernel path and on the fused
+    one (xmc_fp8_kahan_step): a head that ends inside a tile, one that is the whole first chunk with more tiles than
+    quads, and a single chunk whose last rows lie behind the head."""
+    nc, rows, batch, nh = shape
+    case = H.make_case(nc, rows, batch, 81)
     rng = np.random.default_rng(2)
     if ktype == "e5m2":
         k0 = C.e5m2_encode(rng.standard_normal((nh, 768)).astype(np.float32) * 1e-3)
     else:
         k0 = C.bf16_round(rng.standard_normal((nh, 768)).astype(np.float32) * 1e-3)
     seeds = [31337, 5] if mode != "rtn" else None
-    new, kn, gf, gb = run_kahan(case, k0, ktype, nh, gpu, mode, seeds)
+    seeds = None if seeds is None else (seeds + [77, 78])[:nc]
+    new, kn, gf, gb = run_kahan(case, k0, ktype, nh, gpu, mode, seeds, path=path)
+
+    def rand_fn(c, offs):      # the fast mode's words, by global label row
+        return C.fast_sr_words(seeds[c], c * rows + offs // 768, offs % 768)
+
     ref_codes, ref_k, ref_gx, _ = O.fp8_kahan_step(case["chunks"], k0, case["x"], case["labels"], 0.05, nh, kahan_type=ktype,
-                                                   seeds=seeds, sr_mode="rtn" if mode == "rtn" else "reference")
+                                                   seeds=seeds, rand_fn=rand_fn,
+                                                   sr_mode={"rtn": "rtn", "sr_philox": "reference", "sr_fast": "exact"}[mode])
     mism = total = 0
     for a, b in zip(new, ref_codes):
         d = H.e4m3_ulp_distance(a, b)
@@ -334,7 +350,9 @@ def test_head_kahan_parity(gpu, ktype, mode):
     same = new[0][:nh] == ref_codes[0][:nh]
     kf = C.e5m2_decode(kn) if ktype == "e5m2" else kn
     rf = C.e5m2_decode(ref_k) if ktype == "e5m2" else ref_k
-    tol = (2.0 ** -2 if ktype == "e5m2" else 2.0 ** -7) * np.abs(rf) + 1e-7
+    # (one grid step where the fp32 values in front of the cast differ in their last bits: a quarter of the value for
+    # e5m2, whose subnormal step is 2^-16)
+    tol = (2.0 ** -2 if ktype == "e5m2" else 2.0 ** -7) * np.abs(rf) + (2.0 ** -16 if ktype == "e5m2" else 1e-7)
     assert np.all(np.abs(kf - rf)[same] <= tol[same])
     tot_g = C.e4m3_decode(new[0][:nh]).astype(np.float64) + kf
     tot_r = C.e4m3_decode(ref_codes[0][:nh]).astype(np.float64) + rf
@@ -454,6 +472,16 @@ def test_head_kahan_module(gpu):
         assert d.max() <= 1 and (d != 0).mean() < 2e-3
     assert float(xfc.head_kahan.float().abs().max()) > 0            # the buffer picked up the rounding residue
     assert xfc.xfc_forward(tokens).shape == (32, 1000)
+    # a batch that is not a multiple of 16 takes the three-kernel path: same arithmetic, same oracle
+    before = [w.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    k_before = xfc.head_kahan.float().cpu().numpy().copy()
+    lab24 = torch.tensor([[0, 3], [23, 999], [4, 100]], dtype=torch.int32, device=gpu)
+    assert xfc.xfc_forward_backward(tokens[:24], lab24, [0.05]) == 0
+    ref_codes, ref_k, _, _ = O.fp8_kahan_step(before, k_before, tokens[:24].float().cpu().numpy(), lab24.cpu().numpy(), 0.05,
+                                              204, sr_mode="rtn")
+    for w, r in zip(xfc.xfc_weight, ref_codes):
+        d = H.e4m3_ulp_distance(w.view(torch.uint8).cpu().numpy(), r)
+        assert d.max() <= 1 and (d != 0).mean() < 2e-3
     cfg2 = make_cfg("cuda:0", 1000, 2)
     cfg2.training.FP8 = types.SimpleNamespace(using_head_kahan=False, fp8_head_kahan=False, head_ratio=0.2)
     plain = Fp8XMCBCEChunkedHeadKahanLayer(cfg2)                      # no buffer: the fused kernel
