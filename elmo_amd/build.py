@@ -7,6 +7,7 @@ SRC = os.path.join(HERE, "csrc", "xmc_capi.hip")
 OUT = os.path.join(HERE, "libelmo_xmc.so")
 
 SRC_HEAVY = os.path.join(HERE, "csrc", "xmc_fp8_role_heavy.hip")
+SRC_PLAIN = os.path.join(HERE, "csrc", "xmc_fp8_role_plain.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
@@ -15,6 +16,9 @@ HIPCC_FLAGS = [
 # The second translation unit holds the variants of the step kernel whose tile loop is too large for the compiler's
 # default "#pragma unroll" size limit (see the head of that file); everything else keeps the default.
 HEAVY_FLAGS = ["-mllvm", "-pragma-unroll-threshold=1000000"]
+# The third one holds the headline variants of the step kernel, with the instruction scheduler settings that measured
+# best for them (see the head of that file).
+PLAIN_FLAGS = ["-mllvm", "-misched-cluster=0", "-mllvm", "-amdgpu-use-amdgpu-trackers=1"]
 
 
 def source_files():
@@ -50,9 +54,10 @@ def build(verbose=False):
     digest = source_hash()
     tmp = OUT + ".tmp%d" % os.getpid()
     extra = ["-Rpass-analysis=kernel-resource-usage"] if verbose else []
-    objs = [tmp + ".main.o", tmp + ".heavy.o"]
+    objs = [tmp + ".main.o", tmp + ".heavy.o", tmp + ".plain.o"]
     cmds = [[hipcc] + HIPCC_FLAGS + extra + [f'-DXMC_SOURCE_HASH="{digest}"', "-c", SRC, "-o", objs[0]],
-            [hipcc] + HIPCC_FLAGS + HEAVY_FLAGS + extra + ["-c", SRC_HEAVY, "-o", objs[1]]]
+            [hipcc] + HIPCC_FLAGS + HEAVY_FLAGS + extra + ["-c", SRC_HEAVY, "-o", objs[1]],
+            [hipcc] + HIPCC_FLAGS + PLAIN_FLAGS + extra + ["-c", SRC_PLAIN, "-o", objs[2]]]
     procs = [subprocess.Popen(c, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True) for c in cmds]   # side by side
     outs = [p.communicate() for p in procs]
     log = "".join(o[0] + o[1] for o in outs)

@@ -40,10 +40,7 @@ void fill_device_info(int dev) {
   void* sp = nullptr;
   di.scratch_ptr = (di.ok == 1 && hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) == hipSuccess) ? (unsigned char*)sp : nullptr;
   // opt in to the full 160 KiB of LDS once per device
-#define XMC_STEP_LDS(RMODE, WD) \
-  (void)hipFuncSetAttribute((const void*)fp8_step_role_kernel<RMODE, WD, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, RLDS_BYTES)
-  XMC_STEP_LDS(ROUND_RTN, false); XMC_STEP_LDS(ROUND_RTN, true); XMC_STEP_LDS(ROUND_SR_FAST, false); XMC_STEP_LDS(ROUND_SR_FAST, true);
-#undef XMC_STEP_LDS
+  role_plain_set_lds();
   role_heavy_set_lds();
   (void)hipFuncSetAttribute((const void*)fp8_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FWD_LDS);
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<0>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
@@ -281,10 +278,7 @@ static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     if (rest_tiles > 0) {
       const bool wd = weight_decay != 0.f;
       if (round_mode == XMC_ROUND_SR_PHILOX) role_heavy_launch(round_mode, wd, 0, qgrid, stream, p);
-      else if (round_mode == XMC_ROUND_RTN && wd) fp8_step_role_kernel<ROUND_RTN, true, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
-      else if (round_mode == XMC_ROUND_RTN) fp8_step_role_kernel<ROUND_RTN, false, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
-      else if (wd) fp8_step_role_kernel<ROUND_SR_FAST, true, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
-      else fp8_step_role_kernel<ROUND_SR_FAST, false, 0><<<qgrid, QNT, RLDS_BYTES, stream>>>(p);
+      else role_plain_launch(round_mode, wd, qgrid, stream, p);
     }
     if (g_prof_stop) (void)hipEventRecord(g_prof_stop, stream);
     g_prof_start = g_prof_stop = nullptr;

@@ -832,7 +832,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     for (int nn = 0; nn < 3; nn++) dst[(mb * 3 + nn) * 256 + s * 64 + lane] = acc2[mb][nn];
 }
 
-#ifndef XMC_HEAVY_TU
+#ifndef XMC_HEAVY_TU   // compiled once, in the library's main translation unit
 // grad_X = scale * sum over quads of the member partials; writes fp32 and bf16 [batch, 768].  192 workgroups of 128
 // threads: workgroup (block, m, part) covers lanes 128 part.. of the 256 B-wavefront lanes of a step workgroup.
 __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* partial, int nwg, float scale, float* gx_f32,
@@ -880,5 +880,8 @@ __global__ __launch_bounds__(128) void reduce_gx_role_kernel(const floatx4* part
 // (kahan_type 1, 2), defined in xmc_fp8_role_heavy.hip: opt in to the LDS size (once per device); launch.
 void role_heavy_set_lds();
 void role_heavy_launch(int round_mode, bool weight_decay, int kahan_type, int grid, hipStream_t stream, const QuadParams& p);
+// The other variants (round to nearest, fast stochastic rounding), defined in xmc_fp8_role_plain.hip.
+void role_plain_set_lds();
+void role_plain_launch(int round_mode, bool weight_decay, int grid, hipStream_t stream, const QuadParams& p);
 
 }  // namespace xmc
