@@ -261,7 +261,7 @@ static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     p.cnt_base = 0;
     p.acc_init = 0;
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
-        labels_coo, nnz, n_pad, batch, 0, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
+        labels_coo, nnz, n_pad, batch, 0, 0, num_chunks * rows_per_chunk, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
     quad_desc_prep_kernel<<<desc_blocks + (BP * (D / 4) + 255) / 256, 256, (size_t)(n_pad + 257) * 4, stream>>>(
         p, n_pad, (int*)(ws + WS_TILEPTR), desc, desc_blocks, (const unsigned short*)x_bf16, 1.0f / scale_x, ws + WS_XQ,
@@ -559,7 +559,10 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
   if (features != D || batch <= 0 || batch > T_HALVES * BP) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_last_chunk <= 0 || rows_last_chunk > rows_per_chunk) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
-  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1 || nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
+  // a sort key keeps 24 bits for the label: larger label spaces are taken in segments of whole chunks, each with its own
+  // sorted list of the positives that fall into it and labels counted from the segment's first
+  if (rows_per_chunk >= (1 << 24) - 1 || (long long)num_chunks * rows_per_chunk > 0x7FFFFFFFLL) return XMC_ERR_RANGE;
+  if (nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
   if (weight_type != W_E4M3 && weight_type != W_BF16) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && round_mode != XMC_ROUND_SR_PHILOX && round_mode != XMC_ROUND_SR_FAST) return XMC_ERR_MODE;
   if (round_mode != XMC_ROUND_RTN && !seeds) return XMC_ERR_NULL;
@@ -605,14 +608,9 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
   int n_pad = 0;
   if (nnz > 0) { n_pad = 64; while (n_pad < nnz) n_pad <<= 1; }
 
-  // the positives of every 256 batch rows as their own sorted list (the key keeps eight bits for the row)
-  for (int pr = 0; pr < pairs; pr++) {
-    if (n_pad > 0)
-      quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, 256 * pr,
-                                                                            keys + (size_t)pr * MAX_POS, nullptr);
-    tile_ptr_kernel<<<(num_tiles + 1 + 255) / 256, 256, 0, stream>>>(keys + (size_t)pr * MAX_POS, n_pad, rows_per_chunk, tiles_per_chunk,
-                                                                  num_tiles, tile_ptr + pr * tp_stride);
-  }
+  // chunks per segment of the label space: a multiple of the launch group, fewer than 2^24 - 1 labels
+  int seg_chunks = ((1 << 24) - 2) / rows_per_chunk / group * group;
+  if (seg_chunks < group) return XMC_ERR_RANGE;
   // true-FP8 arithmetic with two or four batch halves: FP8 matrix products, the logits of a pair of halves in one pass
   const bool fp8_logits = weight_type == W_E4M3 && quantize_x && halves >= 2 && !loss_out;
   // e4m3 weights, two batch halves, no compensated head: the feature-split update kernel (X^T in registers)
@@ -621,12 +619,28 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
                                                                         fp8_logits ? 1 : 0, split_update ? 1 : 0, xb, xT, gx_total,
                                                                         loss_part, loss_out ? 2 * num_tiles : 0, dp);
   for (int c = 0; c < num_chunks; c += group) {
+    const int seg0 = c / seg_chunks * seg_chunks;   // first chunk of the segment
+    if (c == seg0) {
+      // the segment's positives of every 256 batch rows as their own sorted list (the key keeps eight bits for the row),
+      // and the first key of each of its tiles
+      const int seg_n = seg0 + seg_chunks <= num_chunks ? seg_chunks : num_chunks - seg0;
+      for (int pr = 0; pr < pairs; pr++) {
+        if (n_pad > 0)
+          quad_sort_kernel<<<n_pad / 64, 256, (size_t)(n_pad + 256) * 4, stream>>>(labels_coo, nnz, n_pad, batch, 256 * pr,
+                                                                                seg0 * rows_per_chunk, seg_n * rows_per_chunk,
+                                                                                keys + (size_t)pr * MAX_POS, nullptr);
+        tile_ptr_kernel<<<(seg_n * tiles_per_chunk + 1 + 255) / 256, 256, 0, stream>>>(
+            keys + (size_t)pr * MAX_POS, n_pad, rows_per_chunk, tiles_per_chunk, seg_n * tiles_per_chunk,
+            tile_ptr + pr * tp_stride + seg0 * tiles_per_chunk);
+      }
+    }
     void* w = chunk_ptrs[c];
     const int nch = c + group <= num_chunks ? group : num_chunks - c;                       // chunks of this launch
     const int rows = (nch - 1) * rows_per_chunk + (c + nch == num_chunks ? rows_last_chunk : rows_per_chunk);
     const int rp = (rows + TL - 1) / TL * TL;           // padded rows of this launch (the G buffers use the stride rows_buf)
     const int tiles = rp / TL;
-    const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;
+    const unsigned label0 = (unsigned)c * (unsigned)rows_per_chunk;                  // global: the fast rounding's random words
+    const unsigned label0_seg = (unsigned)(c - seg0) * (unsigned)rows_per_chunk;     // within the segment: the sorted keys
     TiledSeeds sd;
     for (int k = 0; k < T_GROUP; k++)
       sd.s[k] = seeds && k < nch ? (round_mode == XMC_ROUND_SR_FAST ? fast_seed(seeds[c + k]) : seeds[c + k]) : 0u;
@@ -643,7 +657,7 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
       const int nsub = 2 * tiles, lgrid = nsub < di.cus ? nsub : di.cus;
       tiled_logits_fp8_kernel<<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(
           w, rows, nsub, (const unsigned char*)xb + (size_t)hh * BP * D, keys + (size_t)(hh >> 1) * MAX_POS,
-          tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk, label0, glb + hh * g_half, gbl + hh * g_half, g_half);
+          tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk, label0_seg, glb + hh * g_half, gbl + hh * g_half, g_half);
     }
     for (int hh = 0; !fp8_logits && hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
@@ -656,11 +670,11 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
       const int nsub = 2 * tiles;                                   // sub-tiles of 32 label rows
       const int lgrid = nsub < di.cus ? nsub : di.cus;              // persistent: one workgroup per compute unit
       if (weight_type == W_BF16) {
-        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
-        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
       } else {
-        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
-        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0, gl, gb, pbatch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
       }
     }
     // grad_X of the launch's chunks: one pass over W per pair of batch halves, then the fixed-order sums per half

@@ -136,7 +136,10 @@ __device__ __forceinline__ QTile q_desc_full(q_cdesc* desc, int t) {
 // that precede the workgroup's own over a quarter of the set (equal keys: the one that comes first in the input
 // precedes), and the sum of the four counts is the key's position in the output.  Grid: max(1, n_pad / 64) x 256
 // threads, (n_pad + 256) * 4 bytes of LDS.
-__global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, int row0, unsigned* keys, int* flags) {
+// Labels are taken relative to label_base, and those outside [label_base, label_base + label_count) are dropped: a
+// label space of 2^24 labels and more is sorted in segments of whole chunks (a key keeps 24 bits for the label).
+__global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz, int n_pad, int batch, int row0, int label_base,
+                                                        int label_count, unsigned* keys, int* flags) {
   extern __shared__ unsigned sk[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   if (blockIdx.x == 0 && flags)
@@ -155,8 +158,9 @@ __global__ __launch_bounds__(256) void quad_sort_kernel(const int* coo, int nnz,
 #pragma unroll
     for (int u = 0; u < 8; u++) {
       const int i = i0 + u * 256;
-      const int r = e[u].x - row0, lab = e[u].y;
-      if (i < n_pad) sk[i] = (r >= 0 && r < 256 && r + row0 < batch && lab >= 0 && lab < (1 << 24) - 1) ? (((unsigned)lab << 8) | (unsigned)r) : 0xFFFFFFFFu;
+      const int r = e[u].x - row0;
+      const long long lab = (long long)e[u].y - label_base;
+      if (i < n_pad) sk[i] = (r >= 0 && r < 256 && r + row0 < batch && e[u].y >= 0 && lab >= 0 && lab < label_count && lab < (1 << 24) - 1) ? (((unsigned)lab << 8) | (unsigned)r) : 0xFFFFFFFFu;
     }
   }
   __syncthreads();

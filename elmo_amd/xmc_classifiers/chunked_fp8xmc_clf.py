@@ -103,7 +103,10 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self._max_batch = int(_opt(cfg.data, "batch_size", ops.MAX_BATCH))
         if self.fake_fp8_matmul:
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "simulated FP8 has no per-tensor scales"
-        if self.fake_fp8_matmul or self._max_batch > ops.MAX_BATCH:
+        # the fused kernel's sort keys hold 24 bits of label: larger label spaces run on the three-kernel path, which sorts
+        # the positives per segment of the label space
+        self._wide = self.num_labels >= (1 << 24) - 1
+        if self.fake_fp8_matmul or self._max_batch > ops.MAX_BATCH or self._wide:
             self._tiled_workspace = ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device,
                                                               min(max(self._max_batch, ops.MAX_BATCH), ops.MAX_BATCH_TILED))
 
@@ -183,7 +186,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, **extra)
-        elif embed.shape[0] > ops.MAX_BATCH:
+        elif embed.shape[0] > ops.MAX_BATCH or self._wide:
             # the fused kernel holds 128 batch rows; larger batches take the three-kernel path with the same arithmetic
             # (logits from e4m3(X), saturating cast) and the same rounding modes and random words
             assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128"

@@ -199,7 +199,9 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *                    where the final cast does not saturate (NaN above 464)
  *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
- *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row
+ *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row.  The label space may exceed the 2^24 labels
+ *                    the sort keys of xmc_fp8_step hold (up to 2^31 - 1 labels, a chunk below 2^24 - 1 rows): the
+ *                    positives are then sorted once per segment of whole chunks with fewer than 2^24 - 1 labels
  *   round_mode       XMC_ROUND_RTN, XMC_ROUND_SR_PHILOX, or XMC_ROUND_SR_FAST with the random words of xmc_fp8_step's
  *                    mode of that name (bf16 weights: the hardware converter to bf16, which adds the upper 16 bits of the
  *                    word to the fp32 pattern); batch: 1..512, any value (processed in one, two or four halves of 128 rows)

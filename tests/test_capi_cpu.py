@@ -152,3 +152,23 @@ def test_dropout_quantize_rejects_bad_arguments_before_touching_the_device():
     assert call(cols=770) == -2 and call(rows=0) == -2 and call(p=1.0) == -2 and call(p=-0.1) == -2
     assert call(rows=1 << 22, cols=1024) == -4
     assert call(x=P + 4) == -3 and call(x=P + 4, t=1) != -3 and call(out=P + 2) == -3
+
+
+def test_three_kernel_path_accepts_label_spaces_of_2_24_and_more():
+    """The sort key keeps 24 bits for the label; the three-kernel path takes larger label spaces in segments of whole
+    chunks, so 64 chunks of 262,272 rows (16,785,408 labels) pass the range check and fail only on the workspace size
+    given here (no device is touched).  A single chunk of 2^24 rows, and the fused path at this size, are refused."""
+    lib = _lib.load()
+    P = 0x10000
+    nc, rows = 64, 262272
+    assert nc * rows >= 1 << 24
+    arr = (ctypes.c_void_p * nc)(*([P] * nc))
+
+    def tiled(nc_, rows_, wsb):
+        return lib.xmc_tiled_step(arr, nc_, rows_, rows_, 0, P, 32, 768, P, 4, 0.05, None, 0, 1, 1, None, 0, 0, P, None, None,
+                                  P, wsb, None)
+
+    assert tiled(nc, rows, 1024) == -5            # XMC_ERR_WORKSPACE: the label count itself is accepted
+    assert tiled(1, 1 << 24, 1 << 40) == -4       # one chunk must stay below 2^24 rows
+    sarr = (ctypes.c_uint32 * nc)(*([0] * nc))
+    assert lib.xmc_fp8_step(arr, nc, rows, P, 32, 768, P, 4, 0.05, sarr, 0, 1.0, 1.0, P, None, P, 1 << 40, None) == -4

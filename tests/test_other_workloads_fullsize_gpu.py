@@ -128,3 +128,52 @@ def test_bf16_layer_at_131k_labels_against_the_whole_oracle(gpu):
     ref_w, ref_gx, _ = O.bf16_step(w, x, labels, 0.05, cfg.num_chunks, sr_mode="rtn")
     check_bf16_weights(new, ref_w, w, x)
     check_gx(gf, gb, ref_gx)
+
+
+def test_label_space_above_2_24_on_the_three_kernel_path(gpu):
+    """16,785,408 labels (64 chunks of 262,272 rows, 12.9 GB of e4m3 weights), batch 32, true-FP8 arithmetic: the positives
+    are sorted in two segments of the label space (63 chunks + 1).  Positives on both sides of the segment boundary, at
+    label 2^24 and beyond and on the last label; lr = 0 is the identity, grad_X equals library GEMMs over all chunks,
+    sampled rows (among them every row with a positive) equal the oracle after a real step."""
+    import torch
+    from elmo_amd import ops
+    nc, rows, batch = 64, 262272, 32
+    L = nc * rows
+    assert L >= 1 << 24
+    gen = torch.Generator(device=gpu).manual_seed(9)
+    chunks = [(torch.randn(rows, 768, generator=gen, device=gpu) * 0.02).to(torch.float8_e4m3fn) for _ in range(nc)]
+    x_np = synth.make_x(batch, 768, 9)
+    base = synth.make_labels(batch, L, 6.0, 1.0, 9)
+    special = np.array([(0, 63 * rows - 1), (1, 63 * rows), (2, (1 << 24) - 1), (3, 1 << 24), (4, (1 << 24) + 1234), (5, L - 1),
+                        (31, L - 64), (7, 1 << 24), (7, 62 * rows + 5)], dtype=base.dtype)
+    labels_np = np.concatenate([base, special])
+    x = torch.from_numpy(x_np).to(gpu).to(torch.bfloat16)
+    labels = torch.from_numpy(labels_np).to(gpu)
+    ws = ops.alloc_tiled_workspace(nc, rows, gpu, batch)
+    probe = [0, 62, 63]
+    keep = {c: chunks[c].view(torch.uint8).clone() for c in probe}
+    g, gf = ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.0, round_mode="rtn", workspace=ws, want_f32=True,
+                           quantize_x=True, saturate=True)
+    for c in probe:
+        a, b = keep[c], chunks[c].view(torch.uint8)
+        assert bool(((a == b) | (((a | b) & 0x7F) == 0)).all())
+    xq = x.to(torch.float8_e4m3fn).float()
+    ref = torch.zeros(batch, 768, device=gpu, dtype=torch.float64)
+    lab = labels.long()
+    for c, wc in enumerate(chunks):
+        w = wc.float()
+        s = torch.sigmoid((w @ xq.t()).to(torch.bfloat16).float()).to(torch.bfloat16)
+        sel = (lab[:, 1] >= c * rows) & (lab[:, 1] < (c + 1) * rows)
+        s[lab[sel, 1] - c * rows, lab[sel, 0]] -= 1.0
+        ref += (s.float().t() @ w).double()
+        del w, s
+    ref = ref.float()
+    assert (gf - ref).abs().max().item() <= 2e-3 * ref.abs().max().item()
+    sample = np.unique(np.concatenate([sample_rows(labels_np, nc, rows, 4), special[:, 1],
+                                       np.arange(63 * rows - 70, 63 * rows + 70), np.arange((1 << 24) - 70, (1 << 24) + 70)]))
+    before = snapshot(chunks, rows, sample)
+    ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.05, seeds=list(range(nc)), round_mode="rtn", workspace=ws, quantize_x=True,
+                   saturate=True)
+    check_sampled_rows(chunks, rows, sample, before, x_np, labels_np, 0.05)
+    del chunks, ws, keep
+    torch.cuda.empty_cache()
