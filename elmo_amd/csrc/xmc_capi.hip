@@ -246,9 +246,6 @@ static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     p.wd_eff = weight_decay * scale_w;   // T = c - (lr / s) (A + wd s c) for codes c = W / s
     p.batch = batch;
     int qgrid = grid / 32 * 32;   // whole quads on every XCD
-#ifdef XMC_DEV_GRID
-    if (getenv("XMC_STEP_GRID")) qgrid = atoi(getenv("XMC_STEP_GRID"));   // working builds only
-#endif
     if (qgrid < 32) return XMC_ERR_DEVICE;
     p.nquads = qgrid >> 2;
     // with a compensated head the tiles that hold its rows run first, as a launch of their own

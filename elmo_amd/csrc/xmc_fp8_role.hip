@@ -60,6 +60,9 @@ constexpr int RLDS_BYTES = RLDS_M + 256;
 
 static_assert(RLDS_BYTES <= 160 * 1024, "LDS budget");
 
+// Built with -DXMC_TIMING the wavefronts add up the clocks they spend in each phase of an iteration and leave the sums
+// in the unused tail of their quad's exchange slots when the launch ends (the clocks per tile quoted in the profile
+// summaries come from such builds); without it the macros are empty.
 #ifdef XMC_TIMING
 #define RT_DECL unsigned long long rt_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, rt_t0 = 0, rt_t1 = 0; (void)rt_t0; (void)rt_t1
 #define RT_NOW(x) x = __builtin_readcyclecounter()
@@ -119,10 +122,6 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
     }
     s[0] = w01.x + k[0]; s[1] = w01.y + k[1]; s[2] = w23.x + k[2]; s[3] = w23.y + k[3];
   };
-#ifdef XMC_X_NOUPDATE
-  if (c == 7 && ab[0][0] + ab[1][1] + ab[2][2] == 1.2345f) *(volatile unsigned*)bl.dummy = wq[0] + wq[1] + wq[2];
-  return;
-#endif
   if (c < 3) {
     const int cg = c;
     const unsigned wv = wq[cg];
@@ -209,11 +208,7 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
       // the block's 12 bytes per lane go to the image of updated weights in LDS (rows of 192 bytes);
       // the image is stored to memory as whole 192-byte row segments in the next iteration
       typedef unsigned uintx3 __attribute__((ext_vector_type(3)));
-#ifndef XMC_X_NOSTORE
       *(__attribute__((address_space(3))) uintx3*)(lds + oimg + bl.orow_lane + 16 * nb * QCOLS) = uintx3{outw[0], outw[1], outw[2]};
-#else
-      if (outw[0] + outw[1] + outw[2] == 0x12345u) *(__attribute__((address_space(3))) unsigned*)(lds + oimg) = 1;
-#endif
     }
   }
 }
@@ -307,22 +302,16 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     auto wcol_piece = [&](int slot, const QTile& q, int s) {
       if (a + 4 * s >= 13) return;
       const unsigned off = q.rows_valid == TL ? woff_full[s] : wcol_offset(s, q.rows_valid - 1);
-#ifndef XMC_X_NOLOADS
       q_lds_load16_sbase(q.base, off, (unsigned)(RLDS_C + slot * QWC_BYTES + (a + 4 * s) * 1024));
-#endif
     };
     auto rows_piece = [&](int slot, const QTile& q, int s) {
       if (ra + 4 * s >= 13) return;
       const unsigned off = q.rows_valid == TL ? roff_full[s] : rows_offset(s, q.rows_valid - 1);
-#ifndef XMC_X_NOLOADS
       if (ra + 4 * s == 12) {   // the last piece is half a piece: 32 chunks
         if (lane < 32) q_lds_load16_sbase(q.base, off, (unsigned)(RLDS_R + slot * RROW_BYTES + 12 * 1024));
       } else {
         q_lds_load16_sbase(q.base, off, (unsigned)(RLDS_R + slot * RROW_BYTES + (ra + 4 * s) * 1024));
       }
-#else
-      q_lds_load4_l2(srcflags, (unsigned)(RLDS_M + 192));   // keeps the count of operations the waits are written for
-#endif
     };
     auto rows_pieces = [&](int slot, const QTile& q) {
 #pragma unroll
@@ -331,12 +320,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     // block a (the part member a produced) of the G tile of position t, four pieces of 1 KiB, a linear copy
     const unsigned gsrc_lane = (unsigned)(a * 4096 + lane * 16);
     auto gather = [&](int t, int buf) {
-#ifndef XMC_X_NOLOADS
 #pragma unroll
       for (int s = 0; s < 4; s++)
         q_lds_load16_l2_sbase(exq + (t & (QSLOTS - 1)) * QG_BYTES + s * 1024, gsrc_lane,
                               (unsigned)(RLDS_G + buf * RG_BYTES + a * 4096 + s * 1024));
-#endif
     };
     // the four counters of member a's wavefronts, as they are now, into LDS (read in the next iteration)
     auto issue_snapshot = [&](int i) {
@@ -405,7 +392,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       // time; a key costs vector instructions only if it lies in this wavefront's block (label rows 16m.., batch rows
       // 32a..).  Up to seven keys behind the tile's last are read and ignored; the buffer behind the keys belongs to
       // the workspace.
-#ifndef XMC_X_NOPOS
       if (q.p1 > q.p0) {
         float sg[2][4];
 #pragma unroll
@@ -440,7 +426,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
           sb[blk][1] = bf16_pack2(sg[blk][2], sg[blk][3]);
         }
       }
-#endif
       if (q.rows_valid < TL) {   // rows past the end of the chunk contribute nothing
 #pragma unroll
         for (int blk = 0; blk < 2; blk++)
@@ -527,13 +512,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       const bool do_a = i + RQ < n_it;
       const int wslot = w0 == 0 ? RC_RING - 1 : w0 - 1;   // (i + RQ) % RC_RING
       floatx4 z[2];
-#ifndef XMC_X_NOSTAGEA
       stage_a_logits(sa, z, [&](int ks) { if (ks < 4) wcol_piece(wslot, qa, ks); });
-#else
-      z[0] = z[1] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) wcol_piece(wslot, qa, ks);
-#endif
       // the counters as they are now, for the next iteration; everything behind this point may stay in flight over the
       // barrier
       issue_snapshot(i);
@@ -564,11 +543,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       qr_n = q_desc_head(cdesc, tile_at(i + 1 + RQ + RR_RING - 1));
       qb_n = q_desc_full(cdesc, tile_at(i + 1));
       RT_NOW(rt_t1); RT_ADD(3, rt_t0, rt_t1);
-#ifndef XMC_X_NOSTAGEA
       if (do_a) stage_a_finish(i + RQ, qa, z);
-#else
-      if (do_a) { unsigned char* dst = gdst_lane + ((i + RQ) & (QSLOTS - 1)) * QG_BYTES; *(uint2*)dst = uint2{0u, 0u}; *(uint2*)(dst + 512) = uint2{0u, 0u}; }
-#endif
       RT_NOW(rt_t0); RT_ADD(4, rt_t1, rt_t0);
       // ---- the update of those blocks, with the rows of position i + RQ + 2 (the only loads that miss the L2) requested
       //      between its pieces
@@ -616,9 +591,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 
   // ============================================================================================= B wavefronts
   const int s = f;       // features 192m + 48s .. +47
-#ifdef XMC_X_BPRIO
-  __builtin_amdgcn_s_setprio(3);
-#endif
   floatx4 acc2[8][3];    // grad_X[128 batch rows x 48 features]
   {
     // a second launch of a step continues the sums of the first
@@ -657,13 +629,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   auto so_store = [&](const QTile& qp, int jj, const intx4& ov) {
     typedef __attribute__((address_space(1))) intx4 gi4;
     unsigned char* dst = so_row[jj] < qp.rows_valid ? qp.base + so_mem[jj] : bl.dummy;
-#ifndef XMC_X_NOSTORE
     // plain stores on purpose: non-temporal ones keep the exchanged G tiles and the tiles between their two fetches in
     // the XCD's L2 (reads from memory drop from 1.34 to 1.05 times the weights) but cost 5 % of the kernel's time
     *(gi4*)(unsigned long long)dst = ov;
-#else
-    if (ov.x == 0x12345) *(gi4*)(unsigned long long)dst = ov;
-#endif
   };
   auto store_out = [&](const QTile& qp, int slot) {
     intx4 ov[3];
@@ -742,11 +710,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     for (int k = 0; k < NS; k++) {
       if ((k & 7) == 1 && k < 24) so_v = so_read((i + 1) & 1, k >> 3);
       if ((k & 7) == 5 && k < 24) so_store(q_p, k >> 3, so_v);
-#ifndef XMC_X_NOBLDS
       request(k + PD);
-#else
-      if (k + PD < NS) op[k + PD] = op[k & 1];
-#endif
       // vector pieces of this step
       if (k == 0) {
 #pragma unroll
@@ -803,9 +767,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
 #pragma unroll
         for (int nn = 0; nn < 3; nn++) acc2[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(op[k], wb[ks2][nn], acc2[mb][nn], 0, 0, 0);
       }
-#ifndef XMC_X_NOBFENCE
       QFENCE();
-#endif
     }
     if (NBB == 4) {
 #pragma unroll
