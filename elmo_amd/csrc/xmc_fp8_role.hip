@@ -60,21 +60,6 @@ constexpr int RLDS_BYTES = RLDS_M + 256;
 
 static_assert(RLDS_BYTES <= 160 * 1024, "LDS budget");
 
-// Built with -DXMC_TIMING the wavefronts add up the clocks they spend in each phase of an iteration and leave the sums
-// in the unused tail of their quad's exchange slots when the launch ends (the clocks per tile quoted in the profile
-// summaries come from such builds); without it the macros are empty.
-#ifdef XMC_TIMING
-#define RT_DECL unsigned long long rt_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, rt_t0 = 0, rt_t1 = 0; (void)rt_t0; (void)rt_t1
-#define RT_NOW(x) x = __builtin_readcyclecounter()
-#define RT_ADD(k, from, to) rt_acc[k] += (to) - (from)
-#define RT_DUMP(wave) do { if (lane == 0) { unsigned long long* d_ = (unsigned long long*)(exq + (size_t)(m * 2 + ((wave) >> 2)) * QG_BYTES + RG_BYTES + ((wave) & 3) * 1024); \
-    for (int k_ = 0; k_ < 8; k_++) d_[k_] = rt_acc[k_]; } } while (0)
-#else
-#define RT_DECL
-#define RT_NOW(x)
-#define RT_ADD(k, from, to)
-#define RT_DUMP(wave)
-#endif
 
 // row permutation within sixteen rows of the G image: rows 8..11 and 12..15 trade places, so that the four row groups
 // a transposing read touches (rows 8kg..8kg+3) fall into different halves of the LDS banks
@@ -483,16 +468,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     QTile qa_n = q_desc_full(cdesc, tile_at(RQ)), qr_n = q_desc_head(cdesc, tile_at(RQ + RR_RING - 1)), qb_n = q_desc_full(cdesc, tile_at(0));
     int sa = RQ % RR_RING;    // (i + RQ) % RR_RING, the rows image stage A reads
     int w0 = 0;               // i % RC_RING
-    RT_DECL;
-    RT_NOW(rt_t0);
-#ifdef XMC_TIMING
-    const unsigned long long rt_begin = rt_t0;
-#endif
     for (int i = 0; i < n_it; i++) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      RT_NOW(rt_t0);
       __syncthreads();
-      RT_NOW(rt_t1); RT_ADD(1, rt_t0, rt_t1);
       const QTile qa = qa_n, qr = qr_n, qb = qb_n;
       const int abort_word = *(const lds_int*)(lds + abort_base + ((i + 1) & 1) * 4);
       // the counters as they were in the middle of the iteration before
@@ -501,13 +479,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       if (i + 1 < n_it) {
         const int fmin = min(min((int)__builtin_amdgcn_readfirstlane(fl.x), (int)__builtin_amdgcn_readfirstlane(fl.y)),
                              min((int)__builtin_amdgcn_readfirstlane(fl.z), (int)__builtin_amdgcn_readfirstlane(fl.w)));
-#ifdef XMC_TIMING
-        if (fmin < i + 2) rt_acc[6]++;
-#endif
         wait_published(i + 2, fmin, i);
         gather(i + 1, (i + 1) & 1);
       }
-      RT_NOW(rt_t0); RT_ADD(2, rt_t1, rt_t0);
       // ---- stage A of position i + RQ, the columns of the same tile requested between its matrix instructions
       const bool do_a = i + RQ < n_it;
       const int wslot = w0 == 0 ? RC_RING - 1 : w0 - 1;   // (i + RQ) % RC_RING
@@ -542,9 +516,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       qa_n = q_desc_full(cdesc, tile_at(i + 1 + RQ));
       qr_n = q_desc_head(cdesc, tile_at(i + 1 + RQ + RR_RING - 1));
       qb_n = q_desc_full(cdesc, tile_at(i + 1));
-      RT_NOW(rt_t1); RT_ADD(3, rt_t0, rt_t1);
       if (do_a) stage_a_finish(i + RQ, qa, z);
-      RT_NOW(rt_t0); RT_ADD(4, rt_t1, rt_t0);
       // ---- the update of those blocks, with the rows of position i + RQ + 2 (the only loads that miss the L2) requested
       //      between its pieces
       {
@@ -564,7 +536,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
           }
         if (NBB == 4) rows_pieces(rslot, qr);
       }
-      RT_NOW(rt_t1); RT_ADD(5, rt_t0, rt_t1);
       // Loads and stores complete in order.  Waiting for all but the stores of G and the rows covers the gather, the
       // columns and the snapshot, all issued long before, and everything of the iteration before, whose stores of G can
       // now be published.
@@ -575,17 +546,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
         if (ra == 0) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
       }
-      RT_NOW(rt_t0); RT_ADD(7, rt_t1, rt_t0);
       if (lane == 0) __hip_atomic_store(myflag, min(i + RQ, n_it), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       sa = sa == RR_RING - 1 ? 0 : sa + 1;
       w0 = w0 == RC_RING - 1 ? 0 : w0 + 1;
     }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // the last loads still target LDS
     __syncthreads();   // the last tile's updated weights are in LDS: the B wavefronts store them
-#ifdef XMC_TIMING
-    RT_NOW(rt_t1); rt_acc[0] = rt_t1 - rt_begin;
-#endif
-    RT_DUMP(a);
     return;
   }
 
@@ -645,16 +611,9 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   q_p.rows_valid = 0;   // no previous tile yet: the first iteration's stores all go to the dummy place
   int w0 = 0;   // i % RC_RING
   int n_done = 0;
-  RT_DECL;
-  RT_NOW(rt_t0);
-#ifdef XMC_TIMING
-  const unsigned long long rt_begin = rt_t0;
-#endif
   for (int i = 0; i < n_it; i++) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    RT_NOW(rt_t0);
     __syncthreads();
-    RT_NOW(rt_t1); RT_ADD(1, rt_t0, rt_t1);
     const QTile q = q_n;
     const unsigned oimg = (unsigned)(RLDS_O + (i & 1) * RO_BYTES);
     const unsigned wc = (unsigned)(RLDS_C + w0 * QWC_BYTES);
@@ -695,7 +654,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     if (__builtin_amdgcn_readfirstlane(abort_word) != 0) break;
     n_done = i + 1;
     bf16x8 wb[2][3];
-    RT_NOW(rt_t0); RT_ADD(2, rt_t1, rt_t0);
 
     floatx4 aa[2][3];       // A^T of the block in progress and of the one being rounded
     unsigned wq[2][3];      // their old weights
@@ -776,15 +734,10 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     q_p = q;
     q_n = q_desc_full(cdesc, tile_at(i + 1));
     w0 = w0 == RC_RING - 1 ? 0 : w0 + 1;
-    RT_NOW(rt_t1); RT_ADD(3, rt_t0, rt_t1);
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __syncthreads();   // every wavefront has written its part of the last tile's image
   if (n_done > 0) store_out(q_p, (n_done + 1) & 1);
-#ifdef XMC_TIMING
-  RT_NOW(rt_t1); rt_acc[0] = rt_t1 - rt_begin;
-#endif
-  RT_DUMP(v);
 
   // ---- per-workgroup grad_X partial, summed in a fixed order by reduce_gx_role_kernel: [24 blocks][4 B wavefronts][64 lanes]
   floatx4* dst = p.partial + (size_t)g * 24 * 256;
