@@ -84,7 +84,7 @@ int check_common(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, co
   if (features != D || batch <= 0 || batch > BP || batch % 16 != 0) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
-  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1) return XMC_ERR_RANGE;
+  if ((long long)num_chunks * rows_per_chunk > 0x7FFFFFFFLL) return XMC_ERR_RANGE;   // the fused step has a lower limit of its own
   for (int c = 0; c < num_chunks; c++) {
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
@@ -194,6 +194,8 @@ static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
                       void* grad_x_bf16, float* grad_x_f32, void* workspace, size_t workspace_bytes, void* stream_) {
   int st = check_common(chunk_ptrs, num_chunks, rows_per_chunk, x_bf16, batch, features, workspace, workspace_bytes);
   if (st != XMC_OK) return st;
+  // a sort key keeps 24 bits for the label (xmc_tiled_step takes larger label spaces in segments)
+  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1) return XMC_ERR_RANGE;
   if (!grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
   if (((uintptr_t)labels_coo & 7) != 0) return XMC_ERR_ALIGN;   // read as (row, label) pairs
   if (nnz < 0 || nnz > MAX_POS) return XMC_ERR_RANGE;
@@ -325,7 +327,7 @@ int xmc_fp8_forward_static(void* const* chunk_ptrs, int num_chunks, int rows_per
   if (features != D || batch <= 0 || batch > BP || batch % 16 != 0) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_per_chunk % 16 != 0) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
-  if ((long long)num_chunks * rows_per_chunk >= (1LL << 24) - 1) return XMC_ERR_RANGE;
+  if ((long long)num_chunks * rows_per_chunk > 0x7FFFFFFFLL) return XMC_ERR_RANGE;
   for (int c = 0; c < num_chunks; c++) {
     if (!chunk_ptrs[c]) return XMC_ERR_NULL;
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;

@@ -175,5 +175,22 @@ def test_label_space_above_2_24_on_the_three_kernel_path(gpu):
     ops.tiled_step(chunks, rows, "e4m3", x, labels, 0.05, seeds=list(range(nc)), round_mode="rtn", workspace=ws, quantize_x=True,
                    saturate=True)
     check_sampled_rows(chunks, rows, sample, before, x_np, labels_np, 0.05)
-    del chunks, ws, keep
+    # inference over the same label space: dense logits (columns around 2^24 and the last ones against a library GEMM on
+    # those rows) and the top-10 without the dense logits
+    x16 = x[:16].contiguous()
+    out = ops.fp8_forward(chunks, x16, L - 5)
+    assert out.shape == (16, L - 5)
+    cols = np.unique(np.concatenate([np.arange((1 << 24) - 40, (1 << 24) + 40), np.arange(L - 45, L - 5), np.arange(0, 40),
+                                     np.arange(63 * rows - 20, 63 * rows + 20)]))
+    wsel = torch.stack([chunks[int(c) // rows][int(c) % rows] for c in cols]).float()
+    ref_z = (x16.to(torch.float8_e4m3fn).float() @ wsel.t()).to(torch.bfloat16)
+    got_z = out[:, torch.from_numpy(cols).to(gpu)]
+    H.assert_bf16_close(got_z.float().cpu().numpy(), ref_z.float().cpu().numpy())
+    vals, idx = ops.fp8_forward_topk(chunks, x16, L - 5, 10)
+    tv, ti = out.float().topk(10, dim=1)
+    assert torch.equal(vals.float(), tv)
+    unique = (tv[:, 1:-1] != tv[:, :-2]) & (tv[:, 1:-1] != tv[:, 2:])       # bf16 logits tie often: compare the untied entries
+    assert torch.equal(idx[:, 1:-1][unique], ti[:, 1:-1][unique]) and int(unique.sum()) > 40
+    assert int(idx.max()) < L - 5
+    del chunks, ws, keep, out
     torch.cuda.empty_cache()
