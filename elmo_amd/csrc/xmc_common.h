@@ -47,7 +47,7 @@ constexpr int QF_XCC = 1024;
 constexpr int QF_ERR = 2044;
 constexpr int QF_STICKY = 2047;
 
-// The quad kernel assumes that workgroup g runs on XCD g % 8, and builds quads of four workgroups with equal g % 8:
+// The step kernel assumes that workgroup g runs on XCD g % 8, and builds quads of four workgroups with equal g % 8:
 // member m of quad q is workgroup ((q / 8) * 4 + m) * 8 + q % 8.
 __host__ __device__ inline int quad_member_workgroup(int quad, int m) { return (((quad >> 3) << 2) + m) * 8 + (quad & 7); }
 // true if the four members of `quad` did not all record the same XCC id

@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void quad_desc_prep_kernel(const QuadParams p,
   }
 }
 
-// Operand images of X for the quad kernel.
+// Operand images of X for the step kernel.
 //   xq: e4m3(X / scale_x) in v_mfma 16x16x128 B-operand order: operand index ((b/16)*6 + ks), lane = (b%16) + 16*kg,
 //       bytes 0..15: Xq[b][k = 128ks + 16kg + j], bytes 16..31: Xq[b][k = 128ks + 64 + 16kg + (j - 16)] (the order in which
 //       stage A reads the weight rows from LDS)
