@@ -631,7 +631,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     // The operand of step k + 3 is requested in step k.  The vector work of the update of block o (12 weights per lane,
     // eight pieces) is spread over the steps behind the block's last, so that it issues between the matrix instructions.
     constexpr int NS = 16 + 4 * NBB, NALT = 8 * NBB;
-    constexpr int PD = XMC_PD;   // operands are requested this many steps ahead
+    constexpr int PD = KT != 0 ? 2 : XMC_PD;   // operands are requested this many steps ahead (the head-Kahan variants
+                                               // have no registers for a third operand in flight)
     bf16x8 op[NS + PD];
     auto request = [&](int k) {
       if (k >= NS) return;
