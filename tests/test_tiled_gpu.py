@@ -314,13 +314,14 @@ def run_kahan(case, k0, ktype, nh, device, mode, seeds, lr=0.05, path="tiled"):
 
 
 @pytest.mark.parametrize("path,shape", [("tiled", (2, 512, 32, 208)), ("fused", (2, 512, 32, 208)),
-                                        ("fused", (3, 8192, 128, 8192)), ("fused", (1, 4096, 48, 4001))])
+                                        ("fused", (3, 8192, 128, 8192)), ("fused", (1, 4096, 48, 4001)),
+                                        ("fused", (1, 2048, 32, 2048))])
 @pytest.mark.parametrize("ktype,mode", [("bf16", "rtn"), ("bf16", "sr_philox"), ("e5m2", "rtn"), ("bf16", "sr_fast"),
                                         ("e5m2", "sr_fast")])
 def test_head_kahan_parity(gpu, ktype, mode, path, shape):
     """True-FP8 arithmetic with the compensated head (fuse_kernel.py:202-262) on the three-kernel path and on the fused
     one (xmc_fp8_kahan_step): a head that ends inside a tile, one that is the whole first chunk with more tiles than
-    quads, and a single chunk whose last rows lie behind the head."""
+    quads, a single chunk whose last rows lie behind the head, and a layer that is all head (no second launch)."""
     nc, rows, batch, nh = shape
     case = H.make_case(nc, rows, batch, 81)
     rng = np.random.default_rng(2)
