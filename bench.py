@@ -124,7 +124,7 @@ def bench_tiled(args, cfg):
     torch.cuda.empty_cache()
     torch.cuda.reset_peak_memory_stats()
     base_alloc = torch.cuda.memory_allocated()
-    ws = ops.alloc_tiled_workspace(len(views), rows, dev, cfg.batch)
+    ws = ops.alloc_tiled_workspace(len(views), rows, dev, cfg.batch, cfg.dim)
     grad = torch.empty(cfg.batch, cfg.dim, dtype=torch.bfloat16, device=dev)
     true_fp8 = not bf16 and "simfp8" not in cfg.name
     rng = np.random.default_rng(cfg.seed)
@@ -292,7 +292,7 @@ def main():
     cfg = synth.CONFIGS[args.config]
     args.round_given = args.round is not None
     if args.round is None:   # the first workload is defined with round-to-nearest, the others with stochastic rounding
-        args.round = "rtn" if args.config == "cfg1_bf16_131k" else "sr_fast"
+        args.round = "rtn" if args.config.startswith("cfg1_bf16_131k") else "sr_fast"
     if cfg.batch > ops.MAX_BATCH_TILED:
         print(f"bench.py: config {cfg.name} is not runnable by this build (batch > {ops.MAX_BATCH_TILED})", file=sys.stderr)
         sys.exit(2)

@@ -47,21 +47,29 @@ void fill_device_info(int dev) {
   (void)hipFuncSetAttribute((const void*)fp8_forward_select_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, SEL_LDS);
   (void)hipFuncSetAttribute((const void*)quad_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 256) * 4);
   (void)hipFuncSetAttribute((const void*)quad_desc_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (MAX_POS + 257) * 4);
-  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 2>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
-  (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3>::LDS);
+#define XMC_TILED_ATTR(DD)                                                                                                                        \
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 1, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 1, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 1, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 1, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_BF16, 2, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_BF16, 2, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_gradx_kernel<W_E4M3, 2, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TgxGeom<W_E4M3, 2, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, true, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_BF16, false, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_BF16, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, true, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_logits_kernel<W_E4M3, false, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3, DD>::LDS); \
+  (void)hipFuncSetAttribute((const void*)tiled_logits_fp8_kernel<DD>, hipFuncAttributeMaxDynamicSharedMemorySize, TlgGeom<W_E4M3, DD>::LDS)
+  XMC_TILED_ATTR(D);
+  XMC_TILED_ATTR(1024);
+#undef XMC_TILED_ATTR
   (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_RTN>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
   (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_PHILOX>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
   (void)hipFuncSetAttribute((const void*)tiled_update2_kernel<ROUND_SR_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * TU2_GBUF);
   // the update kernels with two batch halves keep 96 KiB of operands in LDS, more than the default limit
-#define XMC_UPD_ATTR(WTYPE, RMODE, KH) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2))
+#define XMC_UPD_ATTR_D(WTYPE, RMODE, KH, DD) (void)hipFuncSetAttribute((const void*)tiled_update_kernel<WTYPE, RMODE, 2, KH, DD>, hipFuncAttributeMaxDynamicSharedMemorySize, tup_lds_bytes(2, DD))
+#define XMC_UPD_ATTR(WTYPE, RMODE, KH) XMC_UPD_ATTR_D(WTYPE, RMODE, KH, D); XMC_UPD_ATTR_D(WTYPE, RMODE, KH, 1024)
   XMC_UPD_ATTR(W_BF16, ROUND_RTN, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_BF16, ROUND_SR_FAST, false);
   XMC_UPD_ATTR(W_E4M3, ROUND_RTN, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, false); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, false);
   XMC_UPD_ATTR(W_E4M3, ROUND_RTN, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_PHILOX, true); XMC_UPD_ATTR(W_E4M3, ROUND_SR_FAST, true);
+#undef XMC_UPD_ATTR_D
 #undef XMC_UPD_ATTR
   g_device_info[dev] = di;
 }
@@ -527,13 +535,18 @@ int xmc_profile_events(void* start_event, void* stop_event) {
 }
 
 size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_batch) {
+  return xmc_tiled_workspace_bytes_ex(num_chunks, rows_per_chunk, max_batch, D);
+}
+
+size_t xmc_tiled_workspace_bytes_ex(int num_chunks, int rows_per_chunk, int max_batch, int features) {
+  if (features != D && features != 1024) return 0;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS || rows_per_chunk <= 0 || max_batch <= 0 || max_batch > T_HALVES * BP) return 0;
   const size_t rows_pad = ((size_t)rows_per_chunk + TL - 1) / TL * TL;
   const size_t tiles = (size_t)num_chunks * (rows_pad / TL);
   const size_t halves = (size_t)tiled_halves(max_batch), pairs = (halves + 1) / 2;
   const size_t rows_buf = (size_t)tiled_group(num_chunks, rows_per_chunk) * rows_pad;   // rows of one launch
   // per batch half G in both orientations; tile_ptr per pair of halves (padded to 64 entries); two loss shares per tile
-  return tiled_layout((int)halves).g + halves * 2 * rows_buf * BP * 2 + pairs * ((tiles + 1 + 63) / 64 * 64 * 4) + (tiles * 8 + 255) / 256 * 256;
+  return tiled_layout((int)halves, features).g + halves * 2 * rows_buf * BP * 2 + pairs * ((tiles + 1 + 63) / 64 * 64 * 4) + (tiles * 8 + 255) / 256 * 256;
 }
 
 int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
@@ -546,16 +559,20 @@ int xmc_tiled_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, 
                            grad_x_bf16, grad_x_f32, loss_out, workspace, workspace_bytes, stream_);
 }
 
-int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
-                      const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
-                      const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
-                      int num_head, float weight_decay, float dropout_p, unsigned long long dropout_seed, void* grad_x_bf16,
-                      float* grad_x_f32, float* loss_out, void* workspace, size_t workspace_bytes, void* stream_) {
+}  // extern "C"
+
+// xmc_tiled_step_ex for DD features (768 or 1024)
+template <int DD>
+static int tiled_step_t(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                        const void* x_bf16, int batch, const int32_t* labels_coo, int nnz, float lr,
+                        const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                        int num_head, float weight_decay, float dropout_p, unsigned long long dropout_seed, void* grad_x_bf16,
+                        float* grad_x_f32, float* loss_out, void* workspace, size_t workspace_bytes, void* stream_) {
   if (!chunk_ptrs || !x_bf16 || !workspace || !grad_x_bf16 || (nnz > 0 && !labels_coo)) return XMC_ERR_NULL;
   if (kahan_type < 0 || kahan_type > 2 || (kahan_type != 0 && (weight_type != W_E4M3 || !kahan))) return XMC_ERR_MODE;
   if (kahan_type != 0 && (num_head < 0 || num_head > rows_per_chunk || !aligned16(kahan))) return XMC_ERR_SHAPE;
   if (kahan_type == 0) num_head = 0;
-  if (features != D || batch <= 0 || batch > T_HALVES * BP) return XMC_ERR_SHAPE;
+  if (batch <= 0 || batch > T_HALVES * BP) return XMC_ERR_SHAPE;
   if (rows_per_chunk <= 0 || rows_last_chunk <= 0 || rows_last_chunk > rows_per_chunk) return XMC_ERR_SHAPE;
   if (num_chunks <= 0 || num_chunks > MAX_CHUNKS) return XMC_ERR_RANGE;
   // a sort key keeps 24 bits for the label: larger label spaces are taken in segments of whole chunks, each with its own
@@ -574,7 +591,7 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     if (!aligned16(chunk_ptrs[c])) return XMC_ERR_ALIGN;
   }
   if (!aligned16(x_bf16) || ((uintptr_t)workspace & 255) != 0 || ((uintptr_t)labels_coo & 7) != 0) return XMC_ERR_ALIGN;
-  if (workspace_bytes < xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk, batch)) return XMC_ERR_WORKSPACE;
+  if (workspace_bytes < xmc_tiled_workspace_bytes_ex(num_chunks, rows_per_chunk, batch, DD)) return XMC_ERR_WORKSPACE;
   DeviceInfo di = device_info();
   if (di.ok != 1) return XMC_ERR_DEVICE;
   hipStream_t stream = (hipStream_t)stream_;
@@ -589,10 +606,10 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
   const int group_max = tiled_group(num_chunks, rows_per_chunk);
   int group = kahan_type != 0 ? 1 : group_max;
   for (int c = 0; c + 1 < num_chunks && group > 1; c++)
-    if ((const unsigned char*)chunk_ptrs[c + 1] != (const unsigned char*)chunk_ptrs[c] + (size_t)rows_per_chunk * D * (weight_type == W_BF16 ? 2 : 1))
+    if ((const unsigned char*)chunk_ptrs[c + 1] != (const unsigned char*)chunk_ptrs[c] + (size_t)rows_per_chunk * DD * (weight_type == W_BF16 ? 2 : 1))
       group = 1;
   const size_t rows_buf = (size_t)group_max * rows_pad;               // rows the G buffers hold
-  const TiledLayout lay = tiled_layout(halves);
+  const TiledLayout lay = tiled_layout(halves, DD);
   unsigned short* xb = (unsigned short*)(ws + lay.xb);
   unsigned short* xT = (unsigned short*)(ws + lay.xt);
   unsigned* keys = (unsigned*)(ws + lay.keys);
@@ -613,8 +630,8 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
   // true-FP8 arithmetic with two or four batch halves: FP8 matrix products, the logits of a pair of halves in one pass
   const bool fp8_logits = weight_type == W_E4M3 && quantize_x && halves >= 2 && !loss_out;
   // e4m3 weights, two batch halves, no compensated head: the feature-split update kernel (X^T in registers)
-  const bool split_update = weight_type == W_E4M3 && halves == 2 && kahan_type == 0;
-  tiled_prep_x_kernel<<<(halves * BP * D + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x,
+  const bool split_update = weight_type == W_E4M3 && halves == 2 && kahan_type == 0 && DD == D;
+  tiled_prep_x_kernel<DD><<<(halves * BP * DD + 255) / 256, 256, 0, stream>>>((const unsigned short*)x_bf16, batch, halves, quantize_x,
                                                                         fp8_logits ? 1 : 0, split_update ? 1 : 0, xb, xT, gx_total,
                                                                         loss_part, loss_out ? 2 * num_tiles : 0, dp);
   for (int c = 0; c < num_chunks; c += group) {
@@ -654,14 +671,14 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     float* lp = loss_part + 2 * c * tiles_per_chunk;
     for (int hh = 0; fp8_logits && hh < halves; hh += 2) {
       const int nsub = 2 * tiles, lgrid = nsub < di.cus ? nsub : di.cus;
-      tiled_logits_fp8_kernel<<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(
-          w, rows, nsub, (const unsigned char*)xb + (size_t)hh * BP * D, keys + (size_t)(hh >> 1) * MAX_POS,
+      tiled_logits_fp8_kernel<DD><<<lgrid, 512, TlgGeom<W_E4M3, DD>::LDS, stream>>>(
+          w, rows, nsub, (const unsigned char*)xb + (size_t)hh * BP * DD, keys + (size_t)(hh >> 1) * MAX_POS,
           tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk, label0_seg, glb + hh * g_half, gbl + hh * g_half, g_half);
     }
     for (int hh = 0; !fp8_logits && hh < halves; hh++) {
       unsigned short* gl = glb + hh * g_half;
       unsigned short* gb = gbl + hh * g_half;
-      const unsigned short* xh = xb + (size_t)hh * BP * D;
+      const unsigned short* xh = xb + (size_t)hh * BP * DD;
       const unsigned* kh = keys + (size_t)(hh >> 1) * MAX_POS;                       // this half's pair: its keys,
       const int* tp = tile_ptr + (hh >> 1) * tp_stride + c * tiles_per_chunk;       // its tile_ptr,
       const unsigned brow0 = (unsigned)((hh & 1) * BP);                             // the half's first row within the pair
@@ -669,32 +686,32 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
       const int nsub = 2 * tiles;                                   // sub-tiles of 32 label rows
       const int lgrid = nsub < di.cus ? nsub : di.cus;              // persistent: one workgroup per compute unit
       if (weight_type == W_BF16) {
-        if (loss_out) tiled_logits_kernel<W_BF16, true><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
-        else tiled_logits_kernel<W_BF16, false><<<lgrid, 512, TlgGeom<W_BF16>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_BF16, true, DD><<<lgrid, 512, TlgGeom<W_BF16, DD>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_BF16, false, DD><<<lgrid, 512, TlgGeom<W_BF16, DD>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
       } else {
-        if (loss_out) tiled_logits_kernel<W_E4M3, true><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
-        else tiled_logits_kernel<W_E4M3, false><<<lgrid, 512, TlgGeom<W_E4M3>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        if (loss_out) tiled_logits_kernel<W_E4M3, true, DD><<<lgrid, 512, TlgGeom<W_E4M3, DD>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
+        else tiled_logits_kernel<W_E4M3, false, DD><<<lgrid, 512, TlgGeom<W_E4M3, DD>::LDS, stream>>>(w, rows, nsub, xh, kh, tp, label0_seg, gl, gb, pbatch, brow0, lp);
       }
     }
     // grad_X of the launch's chunks: one pass over W per pair of batch halves, then the fixed-order sums per half
-    const size_t part_half = (size_t)T_SPLITS * 4 * 24 * 256;   // floatx4 elements of one half's partials
+    const size_t part_half = (size_t)T_SPLITS * 4 * (8 * (DD / 256)) * 256;   // floatx4 elements of one half's partials
     const int ggrid = 4 * ((splits + 7) / 8 * 8);
     for (int h0 = 0; h0 < halves; h0 += 2) {
       const unsigned short* gsrc = gbl + h0 * g_half;
       floatx4* pdst = partial + h0 * part_half;
       if (weight_type == W_BF16) {
-        if (halves == 1) tiled_gradx_kernel<W_BF16, 1><<<ggrid, 512, TgxGeom<W_BF16, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_BF16, 2><<<ggrid, 512, TgxGeom<W_BF16, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_BF16, 1, DD><<<ggrid, 512, TgxGeom<W_BF16, 1, DD>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_BF16, 2, DD><<<ggrid, 512, TgxGeom<W_BF16, 2, DD>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       } else {
-        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1><<<ggrid, 512, TgxGeom<W_E4M3, 1>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
-        else tiled_gradx_kernel<W_E4M3, 2><<<ggrid, 512, TgxGeom<W_E4M3, 2>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        if (halves == 1) tiled_gradx_kernel<W_E4M3, 1, DD><<<ggrid, 512, TgxGeom<W_E4M3, 1, DD>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
+        else tiled_gradx_kernel<W_E4M3, 2, DD><<<ggrid, 512, TgxGeom<W_E4M3, 2, DD>::LDS, stream>>>(w, rows, (int)rows_buf, rp, range, cs, spc, gsrc, g_half, pdst, part_half);
       }
     }
     const int nsub_u = tup_threads(halves) / 256;    // tiles a workgroup of the update kernel works on at a time
     const int ugroups = (tiles + TUP_TILES * nsub_u - 1) / (TUP_TILES * nsub_u);   // rounded up to eight: see the kernel's index map
-    const int ugrid = TRED_WAVES * halves / (tup_threads(halves) / 64) + (12 / tup_csteps(halves)) * ((ugroups + 7) / 8 * 8);
+    const int ugrid = tred_waves(DD) * halves / (tup_threads(halves) / 64) + ((DD / 64) / tup_csteps(halves, DD)) * ((ugroups + 7) / 8 * 8);
 #define XMC_LAUNCH_UPDATE_K(WTYPE, RMODE, HV, KH)                                                                               \
-  tiled_update_kernel<WTYPE, RMODE, HV, KH><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV), stream>>>(                           \
+  tiled_update_kernel<WTYPE, RMODE, HV, KH, DD><<<ugrid, tup_threads(HV), (size_t)tup_lds_bytes(HV, DD), stream>>>(                           \
       w, rows, tiles, glb, g_half, xT, lr, wd, sd, cs, saturate, kahan, kahan_type, nh, label0, partial, part_half, nch, spc, range, rp,  \
       weight_type == W_BF16 ? 1 : 0, gx_total)
 #define XMC_LAUNCH_UPDATE_H(WTYPE, RMODE, KH)                                                                                  \
@@ -707,7 +724,7 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     if (split_update) {
       int streams = (tiles + 7) / 8 * 8;
       streams = streams < 128 ? streams : 128;           // two workgroups per compute unit, four per stream
-      const int grid2 = TRED_WAVES * 2 / 4 + 4 * streams;
+      const int grid2 = tred_waves(D) * 2 / 4 + 4 * streams;
 #define XMC_LAUNCH_UPDATE2(RMODE)                                                                                              \
   tiled_update2_kernel<RMODE><<<grid2, 256, 2 * TU2_GBUF, stream>>>(w, rows, tiles, glb, g_half, (const bf16x8*)xT, lr, wd, sd, cs, saturate, \
                                                                     label0, partial, part_half, nch, spc, range, rp, gx_total)
@@ -731,9 +748,27 @@ int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
 #undef XMC_LAUNCH_UPDATE_H
 #undef XMC_LAUNCH_UPDATE_K
   }
-  tiled_finalize_kernel<<<(batch * D + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32, dp);
+  tiled_finalize_kernel<DD><<<(batch * DD + 255) / 256, 256, 0, stream>>>(gx_total, batch, (unsigned short*)grad_x_bf16, grad_x_f32, dp);
   if (loss_out) tiled_loss_kernel<<<1, 256, 0, stream>>>(loss_part, 2 * num_tiles, loss_out);
   return launch_status();
+}
+
+extern "C" {
+
+int xmc_tiled_step_ex(void* const* chunk_ptrs, int num_chunks, int rows_per_chunk, int rows_last_chunk, int weight_type,
+                      const void* x_bf16, int batch, int features, const int32_t* labels_coo, int nnz, float lr,
+                      const uint32_t* seeds, int round_mode, int quantize_x, int saturate, void* kahan, int kahan_type,
+                      int num_head, float weight_decay, float dropout_p, unsigned long long dropout_seed, void* grad_x_bf16,
+                      float* grad_x_f32, float* loss_out, void* workspace, size_t workspace_bytes, void* stream_) {
+  if (features == D)
+    return tiled_step_t<D>(chunk_ptrs, num_chunks, rows_per_chunk, rows_last_chunk, weight_type, x_bf16, batch, labels_coo, nnz, lr, seeds,
+                           round_mode, quantize_x, saturate, kahan, kahan_type, num_head, weight_decay, dropout_p, dropout_seed,
+                           grad_x_bf16, grad_x_f32, loss_out, workspace, workspace_bytes, stream_);
+  if (features == 1024)
+    return tiled_step_t<1024>(chunk_ptrs, num_chunks, rows_per_chunk, rows_last_chunk, weight_type, x_bf16, batch, labels_coo, nnz, lr,
+                              seeds, round_mode, quantize_x, saturate, kahan, kahan_type, num_head, weight_decay, dropout_p,
+                              dropout_seed, grad_x_bf16, grad_x_f32, loss_out, workspace, workspace_bytes, stream_);
+  return XMC_ERR_SHAPE;
 }
 
 int xmc_copy_probe(void* dst, const void* src, size_t bytes, void* stream_) {

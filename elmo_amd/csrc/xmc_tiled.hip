@@ -44,15 +44,15 @@ struct TiledLayout {
   size_t part;   // grad_X partials [halves][T_SPLITS][128*768] fp32
   size_t g;      // per half: G then G^T, rows_pad x 128 bf16 each, in operand order; then tile_ptr per pair, loss shares
 };
-inline TiledLayout tiled_layout(int halves) {
+inline TiledLayout tiled_layout(int halves, int dd = D) {   // dd: features (768 or 1024)
   TiledLayout l;
   const size_t pairs = (size_t)(halves + 1) / 2;
   l.xb = 0;
-  l.xt = l.xb + (size_t)halves * BP * D * 2;
-  l.keys = l.xt + (size_t)halves * BP * D * 2;
+  l.xt = l.xb + (size_t)halves * BP * dd * 2;
+  l.keys = l.xt + (size_t)halves * BP * dd * 2;
   l.gx = l.keys + pairs * MAX_POS * 4 + 256;      // the kernels read up to seven keys past the end of a list
-  l.part = l.gx + (size_t)halves * BP * D * 4;
-  l.g = l.part + (size_t)halves * T_SPLITS * BP * D * 4;
+  l.part = l.gx + (size_t)halves * BP * dd * 4;
+  l.g = l.part + (size_t)halves * T_SPLITS * BP * dd * 4;
   return l;
 }
 
@@ -81,15 +81,17 @@ __device__ __forceinline__ bf16x8 t_load_w8(const void* w, size_t idx) {
 // (per half: [(16-row block)*6 + ks][lane = row % 16 + 16*((k / 32) % 4)][32 bytes], k = 128 ks + 32 (lane / 16) + byte).
 // xt_split (two halves only): xT in the order of tiled_update2_kernel instead, [feature quarter][wavefront][block cg][K step
 // of 32 batch rows, 8 over both halves][lane][8], row 4kq + e of block cg being feature 12kq + 4cg + e of the wavefront's 48.
+// DD: features of the layer (768, or 1024 = 4 x 4 x 64; every kernel of this path takes it as its last template argument).
+template <int DD>
 __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halves, int quantize, int fp8_image, int xt_split,
                                     unsigned short* xb, unsigned short* xT, float* gx_total, float* loss_part, int n_loss,
                                     const DropoutParams dp) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= halves * BP * D) return;
+  if (i >= halves * BP * DD) return;
   gx_total[i] = 0.f;
-  for (int j = i; j < n_loss; j += halves * BP * D) loss_part[j] = 0.f;
-  int b = i / D, k = i - b * D;
-  unsigned short v = b < batch ? dropout_bf16(x[(size_t)b * D + k], (unsigned)i, dp) : (unsigned short)0;
+  for (int j = i; j < n_loss; j += halves * BP * DD) loss_part[j] = 0.f;
+  int b = i / DD, k = i - b * DD;
+  unsigned short v = b < batch ? dropout_bf16(x[(size_t)b * DD + k], (unsigned)i, dp) : (unsigned short)0;
   unsigned short vq = v;
   int code = 0;
   if (quantize) {
@@ -100,18 +102,19 @@ __global__ void tiled_prep_x_kernel(const unsigned short* x, int batch, int halv
   }
   const int half = b >> 7, bh = b & 127;
   if (fp8_image)
-    ((unsigned char*)xb)[(size_t)half * BP * D + ((size_t)((bh >> 4) * 6 + (k >> 7)) * 64 + (bh & 15) + 16 * ((k >> 5) & 3)) * 32 + (k & 31)] =
+    ((unsigned char*)xb)[(size_t)half * BP * DD + ((size_t)((bh >> 4) * (DD / 128) + (k >> 7)) * 64 + (bh & 15) + 16 * ((k >> 5) & 3)) * 32 + (k & 31)] =
         (unsigned char)(code & 0xFF);
   else
-    xb[(size_t)half * BP * D + ((size_t)((bh >> 4) * (D / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
-  // feature k = 192 fbk + 64 c + 16 kgk + 4 q + e sits in row 4 kgk + e of block 12 fbk + 4 c + q: in the update kernel
-  // a lane then owns 16 consecutive features per step c, and the four lanes of a label row 64 consecutive bytes
-  const int fbk = k / 192, r = k - fbk * 192, kgk = (r >> 4) & 3, nn = 4 * (r >> 6) + ((r >> 2) & 3), e = r & 3;
-  if (xt_split) {
+    xb[(size_t)half * BP * DD + ((size_t)((bh >> 4) * (DD / 32) + (k >> 5)) * 64 + (bh & 15) + 16 * ((k >> 3) & 3)) * 8 + (k & 7)] = vq;
+  // feature k = 64 c + 16 kgk + 4 q + e sits in row 4 kgk + e of block 4 c + q: in the update kernel a lane then owns 16
+  // consecutive features per step c of 64 features, and the four lanes of a label row 64 consecutive bytes
+  const int kgk = (k >> 4) & 3, blk = 4 * (k >> 6) + ((k >> 2) & 3), e = k & 3;
+  if (xt_split) {   // (768 features only)
+    const int fbk = k / 192, r = k - fbk * 192;
     const int wq = r / 48, c48 = r - wq * 48, kq = c48 / 12, rem = c48 - kq * 12, cg = rem >> 2, rr = 4 * kq + (rem & 3);
     xT[((size_t)((((fbk * 4 + wq) * 3 + cg) * 8 + (b >> 5)) * 64 + rr + 16 * ((b >> 3) & 3))) * 8 + (b & 7)] = v;
   } else {
-    xT[(size_t)half * BP * D + ((size_t)((fbk * 12 + nn) * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
+    xT[(size_t)half * BP * DD + ((size_t)(blk * (BP / 32) + (bh >> 5)) * 64 + (4 * kgk + e) + 16 * ((bh >> 3) & 3)) * 8 + (bh & 7)] = v;
   }
 }
 
@@ -132,16 +135,18 @@ __global__ void tiled_zero_kernel(float* p, int n) {
 //      _compute_loss of the reference is written to return (chunked.py:57-72), in fp32 and added per sub-tile for a
 //      fixed-order sum.
 constexpr int TLG_ROWS = 32;
-template <int WT> struct TlgGeom {
-  static constexpr int ROWB = WT == W_BF16 ? D * 2 : D;                 // bytes of one weight row
+template <int WT, int DD> struct TlgGeom {
+  static constexpr int ROWB = WT == W_BF16 ? DD * 2 : DD;               // bytes of one weight row
   static constexpr int STRIDE = ROWB + 16;                               // LDS row stride
   static constexpr int SLOTS = STRIDE / 16;                              // 16-byte slots per LDS row, the last one padding
   static constexpr int PIECES = (TLG_ROWS * STRIDE + 1023) / 1024;       // wave-wide direct-to-LDS loads per sub-tile (49 or 25)
   static constexpr int BUF = PIECES * 1024;                              // bytes of one LDS buffer
   static constexpr int PER_WAVE = (PIECES + 7) / 8;                      // loads of wavefront 0 (7 or 4); the others issue at
   static constexpr int PER_WAVE_MIN = PIECES / 8;                        // least this many (6 or 3)
-  static constexpr int STAGE0 = 3 * BUF + 64;                            // 1 KiB per wavefront: its part of G, transposed
-  static constexpr int LDS = STAGE0 + 8 * 1024;                          // three buffers, eight partial sums of the loss, staging
+  static constexpr int NBUF = 3 * BUF + 64 + 8 * 1024 <= 160 * 1024 ? 3 : 2;   // LDS buffers: the loads run NBUF - 1 sub-tiles ahead
+                                                                         // (two buffers for bf16 rows of 1024 features)
+  static constexpr int STAGE0 = NBUF * BUF + 64;                         // 1 KiB per wavefront: its part of G, transposed
+  static constexpr int LDS = STAGE0 + 8 * 1024;                          // the buffers, eight partial sums of the loss, staging
 };
 
 // 16 bytes per lane from global memory straight into LDS at byte offset ldsoff + 16*lane (wave-uniform offset).  Inline
@@ -155,16 +160,17 @@ __device__ __forceinline__ void t_lds_load16(const unsigned char* g, unsigned ld
 // (always, past the end they fetch the last sub-tile again into a buffer nobody reads, so that the count is the same in
 // every step) and then ten stores of G.  The wait at the top of a step leaves in flight what was issued after the
 // loads of the sub-tile it is about to read.
-template <int WT, bool LOSS>
+template <int WT, bool LOSS, int DD>
 __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int rows, int nsub, const unsigned short* xb,
                                                               const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
                                                               unsigned short* glb, unsigned short* gbl, int batch, unsigned brow0,
                                                               float* loss_part) {
-  typedef TlgGeom<WT> G;
+  typedef TlgGeom<WT, DD> G;
+  constexpr int NB = G::NBUF;
   extern __shared__ __attribute__((aligned(16))) unsigned char tlg_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tlg_lds;
   // no static LDS in this kernel: the direct-to-LDS loads address LDS from byte 0
-  __attribute__((address_space(3))) float* wsum = (__attribute__((address_space(3))) float*)(lds + 3 * G::BUF);
+  __attribute__((address_space(3))) float* wsum = (__attribute__((address_space(3))) float*)(lds + NB * G::BUF);
   const int tid = threadIdx.x, v = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
   // the sorted keys and the tile ranges were written by earlier launches: read them through the scalar (constant) path,
   // so that no vector-memory wait of this loop covers them
@@ -192,26 +198,28 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
   const int gs = (int)gridDim.x;
   __attribute__((address_space(3))) unsigned char* stg = lds + G::STAGE0 + v * 1024;
   issue_sub(blockIdx.x, 0);
-  issue_sub(blockIdx.x + gs, 1);
-  // the X operand of this wavefront's batch rows, behind the first two sub-tiles in the memory pipeline
-  bf16x8 xr[D / 32];
+  if (NB == 3) issue_sub(blockIdx.x + gs, 1);
+  // the X operand of this wavefront's batch rows, behind the first sub-tiles in the memory pipeline
+  bf16x8 xr[DD / 32];
 #pragma unroll
-  for (int ks = 0; ks < D / 32; ks++) xr[ks] = *(const bf16x8*)(xb + ((size_t)(v * (D / 32) + ks) * 64 + lane) * 8);
+  for (int ks = 0; ks < DD / 32; ks++) xr[ks] = *(const bf16x8*)(xb + ((size_t)(v * (DD / 32) + ks) * 64 + lane) * 8);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // from here on the loop counts its own operations: nothing is in flight
-  int it = 0, b0 = 0, b2 = 2;   // it % 3, (it + 2) % 3
+  int it = 0, b0 = 0, b2 = NB - 1;   // it % NB, (it + NB - 1) % NB
   for (int st = blockIdx.x; st < nsub; st += gs, it++) {
     // younger than the loads of this sub-tile: the loads of the next one and the stores of up to two steps
-    if (it == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN) : "memory");
-    // (three stores per wavefront and step: two of G^T, one of G)
+    // (three stores per wavefront and step: two of G^T, one of G); with two buffers only the stores of the step before
+    if (NB == 2) {
+      if (it > 0) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    } else if (it == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN) : "memory");
     else if (it == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 3) : "memory");
     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(G::PER_WAVE_MIN + 6) : "memory");
     // range of positives of the enclosing 64-row tile: asked for here, needed after the MFMAs
     const int p0 = ctile_ptr[st >> 1], p1 = ctile_ptr[(st >> 1) + 1];
     __syncthreads();
-    issue_sub(st + 2 * gs, b2);
+    issue_sub(st + (NB - 1) * gs, b2);
     const int buf = b0;
-    b0 = b0 == 2 ? 0 : b0 + 1;
-    b2 = b2 == 2 ? 0 : b2 + 1;
+    b0 = b0 == NB - 1 ? 0 : b0 + 1;
+    b2 = b2 == NB - 1 ? 0 : b2 + 1;
     floatx4 acc[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
     const unsigned abase = (unsigned)(buf * G::BUF + l16 * G::STRIDE + kg * (WT == W_BF16 ? 16 : 8));
     // the LDS reads run three K steps ahead of the MFMAs (everything unrolled: xr must stay in registers)
@@ -224,8 +232,8 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
 #pragma unroll
     for (int ks = 0; ks < 3; ks++) { araw[ks][0] = rd(ks, 0); araw[ks][1] = rd(ks, 1); }
 #pragma unroll
-    for (int ks = 0; ks < D / 32; ks++) {
-      if (ks + 3 < D / 32) { araw[(ks + 3) & 3][0] = rd(ks + 3, 0); araw[(ks + 3) & 3][1] = rd(ks + 3, 1); }
+    for (int ks = 0; ks < DD / 32; ks++) {
+      if (ks + 3 < DD / 32) { araw[(ks + 3) & 3][0] = rd(ks + 3, 0); araw[(ks + 3) & 3][1] = rd(ks + 3, 1); }
       __builtin_amdgcn_sched_barrier(0);   // keep the reads ahead of the MFMAs that do not need them yet
 #pragma unroll
       for (int lb = 0; lb < 2; lb++) {
@@ -323,10 +331,13 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_kernel(const void* w, int
 //      the weights yields the G of 256 batch rows.  Tile loop, positives, rounding and both layouts of G as above; the
 //      products are exact in fp32 either way, only the order of the fp32 sums differs from the bf16 form.
 //      xq: e4m3 image of the pair's X in B-operand order, [half][(16-row block)*6 + ks][lane][32 bytes] (tiled_prep_x_kernel)
+template <int DD>
 __global__ __launch_bounds__(512, 1) void tiled_logits_fp8_kernel(const void* w, int rows, int nsub, const unsigned char* xq,
                                                                   const unsigned* keys, const int* tile_ptr, unsigned label0_chunk,
                                                                   unsigned short* glb, unsigned short* gbl, size_t g_half) {
-  typedef TlgGeom<W_E4M3> G;
+  typedef TlgGeom<W_E4M3, DD> G;
+  static_assert(G::NBUF == 3, "three buffers");
+  constexpr int KS = DD / 128;   // K steps of the FP8 matrix instruction
   extern __shared__ __attribute__((aligned(16))) unsigned char tlg_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tlg_lds;
   const int tid = threadIdx.x, v = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l16 = lane & 15, kg = lane >> 4;
@@ -354,11 +365,11 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_fp8_kernel(const void* w,
   __attribute__((address_space(3))) unsigned char* stg = lds + G::STAGE0 + v * 1024;
   issue_sub(blockIdx.x, 0);
   issue_sub(blockIdx.x + gs, 1);
-  intx8 xr[2][6];   // the e4m3 operands of this wavefront's batch rows in either half
+  intx8 xr[2][KS];   // the e4m3 operands of this wavefront's batch rows in either half
 #pragma unroll
   for (int hf = 0; hf < 2; hf++)
 #pragma unroll
-    for (int ks = 0; ks < 6; ks++) xr[hf][ks] = *(const intx8*)(xq + (size_t)hf * BP * D + ((size_t)(v * 6 + ks) * 64 + lane) * 32);
+    for (int ks = 0; ks < KS; ks++) xr[hf][ks] = *(const intx8*)(xq + (size_t)hf * BP * DD + ((size_t)(v * KS + ks) * 64 + lane) * 32);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // from here on the loop counts its own operations: nothing is in flight
   int it = 0, b0 = 0, b2 = 2;   // it % 3, (it + 2) % 3
   for (int st = blockIdx.x; st < nsub; st += gs, it++) {
@@ -386,8 +397,8 @@ __global__ __launch_bounds__(512, 1) void tiled_logits_fp8_kernel(const void* w,
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) { araw[ks][0] = rd(ks, 0); araw[ks][1] = rd(ks, 1); }
 #pragma unroll
-    for (int ks = 0; ks < 6; ks++) {
-      if (ks + 2 < 6) { araw[(ks + 2) % 3][0] = rd(ks + 2, 0); araw[(ks + 2) % 3][1] = rd(ks + 2, 1); }
+    for (int ks = 0; ks < KS; ks++) {
+      if (ks + 2 < KS) { araw[(ks + 2) % 3][0] = rd(ks + 2, 0); araw[(ks + 2) % 3][1] = rd(ks + 2, 1); }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int lb = 0; lb < 2; lb++)
@@ -477,8 +488,11 @@ __global__ __launch_bounds__(256) void tiled_loss_kernel(const float* loss_part,
 //      With two batch halves (HV = 2) one pass over W serves both: the step's G^T of either half is staged, and the
 //      workgroup's eight wavefronts are four per half; with one half they are four per four batch blocks (two wavefronts
 //      per SIMD either way: one's LDS reads and conversions run under the other's matrix instructions).
-template <int WT, int HV> struct TgxGeom {
-  static constexpr int ROWB = WT == W_BF16 ? 384 : 192;                  // bytes of this workgroup's features in one row
+template <int WT, int HV, int DD> struct TgxGeom {
+  static constexpr int FB = DD / 4;                                       // features of a workgroup (192 or 256)
+  static constexpr int FW = DD / 16;                                      // features of a wavefront (48 or 64)
+  static constexpr int NN = FW / 16;                                      // ... in blocks of 16 (3 or 4)
+  static constexpr int ROWB = WT == W_BF16 ? 2 * FB : FB;                 // bytes of this workgroup's features in one row
   static constexpr int STRIDE = ROWB + 16;                                // LDS row stride
   static constexpr int SLOTS = STRIDE / 16;                               // 16-byte slots per LDS row, the last one padding
   static constexpr int WPIECES = (32 * SLOTS + 63) / 64;                  // wave-wide loads of the W slice (7 or 13)
@@ -495,10 +509,11 @@ template <int WT, int HV> struct TgxGeom {
 //      A launch may cover several chunks that lie one behind the other in memory (cs rows each, a multiple of the tile
 //      height; the last may be shorter): chunk k owns the partial slots k*spc .. k*spc+spc-1, and no label range crosses
 //      a chunk boundary, so that each chunk's sum can be rounded by itself.
-template <int WT, int HV>
+template <int WT, int HV, int DD>
 __global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int rows, int rows_pad, int bound, int range, int cs, int spc,
                                                           const unsigned short* gbl, size_t g_half, floatx4* partial, size_t part_half) {
-  typedef TgxGeom<WT, HV> G;
+  typedef TgxGeom<WT, HV, DD> G;
+  constexpr int NN = G::NN;
   extern __shared__ __attribute__((aligned(16))) unsigned char tgx_lds[];
   __attribute__((address_space(3))) unsigned char* lds = (__attribute__((address_space(3))) unsigned char*)tgx_lds;
   const unsigned lds0 = (unsigned)(size_t)lds;
@@ -511,11 +526,11 @@ __global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int row
   const int ck = split / spc, lbeg = ck * cs + (split - ck * spc) * range;
   const int cend = min((ck + 1) * cs, bound);   // bound: the launch's rows rounded up to a tile
   if (lbeg >= cend) return;                     // the grid is rounded up to eight ranges; a short last chunk has fewer
-  floatx4 acc[G::NMB][3];
+  floatx4 acc[G::NMB][NN];
 #pragma unroll
   for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int nn = 0; nn < NN; nn++) acc[mb][nn] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int lend = min(lbeg + range, cend);
   const int nsteps = (lend - lbeg + 31) >> 5;
   // Every wavefront issues exactly PER_WAVE loads per step (pieces wv, wv + WAVES, ...; indices past the last piece repeat it),
@@ -528,7 +543,7 @@ __global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int row
       if (piece < G::WPIECES) {
         const int ch = min(piece * 64 + lane, 32 * G::SLOTS - 1), row = ch / G::SLOTS, c16 = min(ch - row * G::SLOTS, G::SLOTS - 2);
         const int lr = min(l0 + row, rows - 1);   // rows past the end re-read a valid one (their G is zero)
-        t_lds_load16((const unsigned char*)w + ((size_t)lr * D + 192 * fb) * (WT == W_BF16 ? 2 : 1) + 16 * c16,
+        t_lds_load16((const unsigned char*)w + ((size_t)lr * DD + G::FB * fb) * (WT == W_BF16 ? 2 : 1) + 16 * c16,
                      lds0 + (unsigned)(stage * G::STAGE + piece * 1024));
       } else {
         const int gp = piece - G::WPIECES;   // piece gp & 7 of batch half gp >> 3
@@ -552,16 +567,16 @@ __global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int row
 #pragma unroll
     for (int mb = 0; mb < G::NMB; mb++)
       ga[mb] = *(const __attribute__((address_space(3))) bf16x8*)(gt + hw * 8192 + ((mb0 + mb) * 64 + lane) * 16);
-    bf16x8 wb[3];
+    bf16x8 wb[NN];
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) {
+    for (int nn = 0; nn < NN; nn++) {
       if (WT == W_BF16) {
-        const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * G::STRIDE + (48 * fw + 16 * nn + 4 * (l16 & 3)) * 2);
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 2)) * G::STRIDE + (G::FW * fw + 16 * nn + 4 * (l16 & 3)) * 2);
         tshortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off));
         tshortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) tshortx4*)(wt + off + 4 * G::STRIDE));
         wb[nn] = __builtin_bit_cast(bf16x8, tshortx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
       } else {
-        const unsigned off = (unsigned)((8 * kg + (l16 >> 1)) * G::STRIDE + 48 * fw + 16 * nn + (l16 & 1) * 8);
+        const unsigned off = (unsigned)((8 * kg + (l16 >> 1)) * G::STRIDE + G::FW * fw + 16 * nn + (l16 & 1) * 8);
         const intx2 raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) intx2*)(wt + off));
         wb[nn] = t_fp8x8_to_bf16x8(raw);
       }
@@ -569,57 +584,60 @@ __global__ __launch_bounds__(512) void tiled_gradx_kernel(const void* w, int row
 #pragma unroll
     for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
-      for (int nn = 0; nn < 3; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
+      for (int nn = 0; nn < NN; nn++) acc[mb][nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ga[mb], wb[nn], acc[mb][nn], 0, 0, 0);
     stage = stage == 2 ? 0 : stage + 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the loads past the end still target LDS
-  // acc[mb][nn][e] = C[batch 128hw + 16(mb0 + mb) + 4kg + e][feature 192fb + 48fw + 16nn + l16]
-  floatx4* dst = partial + (size_t)hw * part_half + ((size_t)split * 4 + fb) * 24 * 256;
+  // acc[mb][nn][e] = C[batch 128hw + 16(mb0 + mb) + 4kg + e][feature FB fb + FW fw + 16nn + l16]
+  floatx4* dst = partial + (size_t)hw * part_half + ((size_t)split * 4 + fb) * (8 * NN) * 256;
 #pragma unroll
   for (int mb = 0; mb < G::NMB; mb++)
 #pragma unroll
-    for (int nn = 0; nn < 3; nn++) dst[((mb0 + mb) * 3 + nn) * 256 + fw * 64 + lane] = acc[mb][nn];
+    for (int nn = 0; nn < NN; nn++) dst[((mb0 + mb) * NN + nn) * 256 + fw * 64 + lane] = acc[mb][nn];
 }
 
 // sum of the partials of one chunk and batch half in a fixed order; bf16 weights: the chunk's contribution is rounded to
 // bf16 before it is added to the fp32 total (chunked.py:116).  Work of one wavefront; 384 of them cover a half.  It runs
 // in the first workgroups of the chunk's update launch (the two do not depend on each other), so the sum costs no
 // launch of its own and hides behind the update.
-constexpr int TRED_WAVES = 384;
+constexpr int tred_waves(int dd) { return 8 * (dd / 256) * 16; }   // (slot, feature quarter, wavefront): 384 or 512
+template <int DD>
 __device__ __forceinline__ void tiled_reduce_wave(int widx, int lane, const floatx4* partial, int nchunks, int spc, int cs, int range,
                                                   int bound, int round_bf16, float* gx_total) {
   // (slot, fb, wavefront of the grad_X kernel's layout); eight loads in flight
   const int slot = widx >> 4, fb = (widx >> 2) & 3, wv = widx & 3;
   const int tid = wv * 64 + lane, l16 = lane & 15, kg = lane >> 4;
-  const int mb = slot / 3, nn = slot - mb * 3;
-  const int col = 192 * fb + 48 * wv + 16 * nn + l16;
+  constexpr int NN = DD / 256, SL = 8 * NN;   // blocks of 16 features per wavefront; slots per (split, feature quarter)
+  const int mb = slot / NN, nn = slot - mb * NN;
+  const int col = (DD / 4) * fb + (DD / 16) * wv + 16 * nn + l16;
   floatx4 tot = {0.f, 0.f, 0.f, 0.f};
   for (int ck = 0; ck < nchunks; ck++) {   // the chunks of the launch, each summed (and rounded) by itself
     const int crows = min((ck + 1) * cs, bound) - ck * cs, splits = (crows + range - 1) / range;
-    const floatx4* pc = partial + (size_t)ck * spc * 4 * 24 * 256;
+    const floatx4* pc = partial + (size_t)ck * spc * 4 * SL * 256;
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
     int sp = 0;
     for (; sp + 8 <= splits; sp += 8) {
       floatx4 v[8];
 #pragma unroll
-      for (int x = 0; x < 8; x++) v[x] = pc[(((size_t)(sp + x) * 4 + fb) * 24 + slot) * 256 + tid];
+      for (int x = 0; x < 8; x++) v[x] = pc[(((size_t)(sp + x) * 4 + fb) * SL + slot) * 256 + tid];
 #pragma unroll
       for (int x = 0; x < 8; x++) s += v[x];
     }
-    for (; sp < splits; sp++) s += pc[(((size_t)sp * 4 + fb) * 24 + slot) * 256 + tid];
+    for (; sp < splits; sp++) s += pc[(((size_t)sp * 4 + fb) * SL + slot) * 256 + tid];
 #pragma unroll
     for (int i = 0; i < 4; i++) tot[i] += round_bf16 ? bf16_rt(s[i]) : s[i];
   }
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int b = 16 * mb + 4 * kg + i;
-    gx_total[(size_t)b * D + col] += tot[i];
+    gx_total[(size_t)b * DD + col] += tot[i];
   }
 }
 
+template <int DD>
 __global__ void tiled_finalize_kernel(const float* gx_total, int batch, unsigned short* gx_bf16, float* gx_f32, const DropoutParams dp) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= batch * D) return;
+  if (i >= batch * DD) return;
   const float v = dropout_backward(gx_total[i], (unsigned)i, dp);
   if (gx_f32) gx_f32[i] = v;
   gx_bf16[i] = bf16_bits(v);
@@ -729,31 +747,32 @@ __device__ __forceinline__ void t_update4(floatx4 a, const unsigned* wraw, const
 }
 
 constexpr int TUP_TILES = 4;                       // tiles of 64 label rows that each group of four wavefronts processes
-// A workgroup owns CS steps of 64 features (CS = 3: a feature quarter, with one or two batch halves; CS = 1: 64 features,
-// with four halves) and keeps their X^T operand blocks of every batch half in LDS: 16 KiB per step and half.
-constexpr int tup_csteps(int halves) { return halves <= 2 ? 3 : 1; }
-constexpr int tup_xbytes(int halves) { return tup_csteps(halves) * 4 * (BP / 32) * 1024; }
+// A workgroup owns CS steps of 64 features (768 features: CS = 3, a feature quarter, with one or two batch halves; 1024
+// features: CS = 2; CS = 1: 64 features, with four halves) and keeps their X^T operand blocks of every batch half in LDS:
+// 16 KiB per step and half.
+constexpr int tup_csteps(int halves, int dd = D) { return halves > 2 ? 1 : dd % 192 == 0 ? 3 : 2; }
+constexpr int tup_xbytes(int halves, int dd = D) { return tup_csteps(halves, dd) * 4 * (BP / 32) * 1024; }
 constexpr int tup_threads(int halves) { return halves == 1 ? 256 : 512; }
-constexpr int tup_lds_bytes(int halves) { return halves * tup_xbytes(halves); }
+constexpr int tup_lds_bytes(int halves, int dd = D) { return halves * tup_xbytes(halves, dd); }
 
 // Launched with tup_threads(HALVES) threads and tup_lds(HALVES) bytes of LDS: four wavefronts per tile, so that a
 // compute unit runs at least eight wavefronts with one batch half (three workgroups) as with more (one workgroup of
 // eight wavefronts, two tiles at a time).
 // HALVES (batch halves: 1, 2 or 4) and KAHAN (a compensated head may be present) are template parameters: with run-time
 // branches around the products the compiler issued every LDS operand read right in front of its matrix instruction.
-template <int WT, int MODE, int HALVES, bool KAHAN>
+template <int WT, int MODE, int HALVES, bool KAHAN, int DD>
 __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES == 2 ? 2 : 1) void tiled_update_kernel(
     void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half_stride, const unsigned short* xT, float lr, float wd, TiledSeeds seeds,
     int cs, int saturate, void* kahan, int kahan_type, int num_head, unsigned label0, const floatx4* red_partial, size_t red_part_half,
     int red_nchunks, int red_spc, int red_range, int red_bound, int red_round_bf16, float* red_total) {
   static_assert(!KAHAN || WT == W_E4M3, "the compensated head belongs to the FP8 layer");
   // the first workgroups sum the chunk's grad_X partials (384 wavefronts per batch half), the others update the weights
-  constexpr int CS = tup_csteps(HALVES), XB = tup_xbytes(HALVES), NFB = 12 / CS, WAVES = tup_threads(HALVES) / 64;
-  constexpr int RED_BLOCKS = TRED_WAVES * HALVES / WAVES;
+  constexpr int CS = tup_csteps(HALVES, DD), XB = tup_xbytes(HALVES, DD), NFB = (DD / 64) / CS, WAVES = tup_threads(HALVES) / 64;
+  constexpr int TRED_WAVES = tred_waves(DD), RED_BLOCKS = TRED_WAVES * HALVES / WAVES;
   if ((int)blockIdx.x < RED_BLOCKS) {
     const int widx = (int)blockIdx.x * WAVES + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
-    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
-                      red_range, red_bound, red_round_bf16, red_total + (size_t)hh * BP * D);
+    tiled_reduce_wave<DD>(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
+                      red_range, red_bound, red_round_bf16, red_total + (size_t)hh * BP * DD);
     return;
   }
   extern __shared__ __attribute__((aligned(16))) unsigned char tup_lds[];
@@ -768,7 +787,7 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
   // wavefronts of the workgroup; from global memory every MFMA would fetch its operand through L1 again.
 #pragma unroll
   for (int hh = 0; hh < HALVES; hh++) {
-    const intx4* src = (const intx4*)(xT + (size_t)hh * D * BP + (size_t)fb * (XB / 2));
+    const intx4* src = (const intx4*)(xT + (size_t)hh * DD * BP + (size_t)fb * (XB / 2));
     for (int s = tid; s < XB / 16; s += (int)blockDim.x)
       *(__attribute__((address_space(3))) intx4*)(lds + hh * XB + s * 16) = src[s];
   }
@@ -788,7 +807,7 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
         gf_n[hh][ks] = tile < ntiles ? *(const bf16x8*)(glb + hh * g_half_stride + ((size_t)((tile * 4 + wv) * 4 + ks) * 64 + lane) * 8) : bf16x8{};
 #pragma unroll
     for (int c = 0; c < CS; c++) {
-      const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * D + 64 * (CS * fb + c) + 16 * kg) * (WT == W_BF16 ? 2 : 1));
+      const intx4* src = (const intx4*)((const unsigned char*)w + ((size_t)row * DD + 64 * (CS * fb + c) + 16 * kg) * (WT == W_BF16 ? 2 : 1));
 #pragma unroll
       for (int q = 0; q < WDW / 4; q++) wr_n[c][q] = live ? src[q] : intx4{0, 0, 0, 0};
     }
@@ -821,7 +840,7 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
 #pragma unroll
   for (int c = 0; c < CS; c++) {              // 16 consecutive features of this lane's row at a time
     const int col0 = 64 * (CS * fb + c) + 16 * kg;
-    const size_t idx = (size_t)row * D + col0;
+    const size_t idx = (size_t)row * DD + col0;
     unsigned wr[WDW], wo[WDW], kr[8] = {0, 0, 0, 0, 0, 0, 0, 0}, ko[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int q = 0; q < WDW / 4; q++) {
@@ -870,8 +889,8 @@ __global__ __launch_bounds__(HALVES == 1 ? 256 : 512, HALVES == 1 ? 3 : HALVES =
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         const int wq = WT == W_BF16 ? 2 * q : q, kq = kahan_type == 1 ? 2 * q : q;
-        t_update4<WT, MODE>(acc[q], wr + wq, kr + kq, head, kahan_type, lr, wd, (unsigned)orow * (unsigned)D + (unsigned)(col0 + 4 * q),
-                            (label0 + (unsigned)row) * (unsigned)(D / 4) + (unsigned)((col0 + 4 * q) >> 2), seed, saturate, wo + wq,
+        t_update4<WT, MODE>(acc[q], wr + wq, kr + kq, head, kahan_type, lr, wd, (unsigned)orow * (unsigned)DD + (unsigned)(col0 + 4 * q),
+                            (label0 + (unsigned)row) * (unsigned)(DD / 4) + (unsigned)((col0 + 4 * q) >> 2), seed, saturate, wo + wq,
                             ko + kq);
       }
     }
@@ -907,10 +926,10 @@ __global__ __launch_bounds__(256, 2) void tiled_update2_kernel(
     void* w, int rows, int ntiles, const unsigned short* glb, size_t g_half, const bf16x8* xt2, float lr, float wd, TiledSeeds seeds, int cs,
     int saturate, unsigned label0, const floatx4* red_partial, size_t red_part_half, int red_nchunks, int red_spc, int red_range,
     int red_bound, float* red_total) {
-  constexpr int RED_BLOCKS = TRED_WAVES * 2 / 4;
+  constexpr int TRED_WAVES = tred_waves(D), RED_BLOCKS = TRED_WAVES * 2 / 4;   // (768 features only)
   if ((int)blockIdx.x < RED_BLOCKS) {
     const int widx = (int)blockIdx.x * 4 + ((int)threadIdx.x >> 6), hh = widx / TRED_WAVES;
-    tiled_reduce_wave(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
+    tiled_reduce_wave<D>(widx - hh * TRED_WAVES, (int)threadIdx.x & 63, red_partial + (size_t)hh * red_part_half, red_nchunks, red_spc, cs,
                       red_range, red_bound, 0, red_total + (size_t)hh * BP * D);
     return;
   }

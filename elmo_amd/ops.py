@@ -241,34 +241,40 @@ def dropout_quantize(x, p, seed):
 WEIGHT_TYPES = {"e4m3": 0, "bf16": 1}
 
 
-def tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch=MAX_BATCH):
-    n = _lib.load().xmc_tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch)
+TILED_FEATURES = (768, 1024)   # input widths of the three-kernel path
+
+
+def tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch=MAX_BATCH, features=FEATURES):
+    n = _lib.load().xmc_tiled_workspace_bytes_ex(num_chunks, rows_per_chunk, max_batch, features)
     if n == 0:
         raise _lib.XmcError("unsupported chunk geometry")
     return n
 
 
-def alloc_tiled_workspace(num_chunks, rows_per_chunk, device, max_batch=MAX_BATCH):
-    return torch.empty(tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch), dtype=torch.uint8, device=device)
+def alloc_tiled_workspace(num_chunks, rows_per_chunk, device, max_batch=MAX_BATCH, features=FEATURES):
+    return torch.empty(tiled_workspace_bytes(num_chunks, rows_per_chunk, max_batch, features), dtype=torch.uint8,
+                       device=device)
 
 
 def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=None, round_mode="rtn", workspace=None,
                grad_out=None, want_f32=False, quantize_x=False, saturate=False, kahan=None, num_head=0, loss_out=None,
                weight_decay=0.0, dropout_p=0.0, dropout_seed=0):
     """One training step of the bf16 layer (chunked.py:76-133) or of the simulated-FP8 mode of the FP8 layer
-    (chunked_fp8xmc_clf.py:98-99,110,115-116), three kernels per chunk.  `chunk_views` are contiguous [rows, 768]
-    tensors (views of one weight tensor, or the FP8 layer's chunk parameters): all have rows_per_chunk rows except the
+    (chunked_fp8xmc_clf.py:98-99,110,115-116), three kernels per chunk.  `chunk_views` are contiguous [rows, d]
+    tensors with d = 768 or 1024 (views of one weight tensor, or the FP8 layer's chunk parameters): all have rows_per_chunk rows except the
     last, which may be shorter.  Updated in place; returns grad_input (bf16) or (grad_input, grad_x_fp32).
     e4m3 weights: quantize_x / saturate select the true-FP8 arithmetic (logits from e4m3(X), saturating cast) instead of
-    the simulated one; `kahan` ([num_head, 768] bf16 or float8_e5m2, updated in place) turns on the head-Kahan update of
+    the simulated one; `kahan` ([num_head, d] bf16 or float8_e5m2, updated in place) turns on the head-Kahan update of
     the first num_head rows of chunk 0 (chunked_head_kahan_fp8xmc_clf.py:127-131).  `loss_out` (a float32 device tensor
     with one element) receives the summed binary cross entropy of the step's logits (what chunked.py:57-72 is written
     to compute).  weight_decay, dropout_p, dropout_seed: as in fp8_step."""
     lib = _lib.load()
-    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == FEATURES
+    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.dim() == 2
+    feats = x.shape[1]
+    assert feats in TILED_FEATURES, "the three-kernel path is built for 768 and 1024 input features"
     ktype = 0
     if kahan is not None:
-        assert weight_type == "e4m3" and kahan.is_cuda and kahan.is_contiguous() and kahan.shape == (num_head, FEATURES)
+        assert weight_type == "e4m3" and kahan.is_cuda and kahan.is_contiguous() and kahan.shape == (num_head, feats)
         assert kahan.dtype in (torch.bfloat16, torch.float8_e5m2) and 0 < num_head <= rows_per_chunk
         ktype = 1 if kahan.dtype == torch.bfloat16 else 2
     assert labels.is_cuda and labels.dtype == torch.int32 and labels.is_contiguous()
@@ -279,23 +285,23 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
     nc = len(chunk_views)
     arr = (ctypes.c_void_p * nc)()
     for i, c in enumerate(chunk_views):
-        assert c.is_cuda and c.is_contiguous() and c.dtype in wdt and c.dim() == 2 and c.shape[1] == FEATURES
+        assert c.is_cuda and c.is_contiguous() and c.dtype in wdt and c.dim() == 2 and c.shape[1] == feats
         assert c.shape[0] == rows_per_chunk or (i == nc - 1 and 0 < c.shape[0] <= rows_per_chunk)
         arr[i] = c.data_ptr()
     batch = x.shape[0]
     assert 0 < batch <= MAX_BATCH_TILED, "batch must be at most 512"
-    if workspace is None or workspace.numel() < tiled_workspace_bytes(nc, rows_per_chunk, batch):
-        workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device, batch)
+    if workspace is None or workspace.numel() < tiled_workspace_bytes(nc, rows_per_chunk, batch, feats):
+        workspace = alloc_tiled_workspace(nc, rows_per_chunk, x.device, batch, feats)
     if grad_out is None:
-        grad_out = torch.empty(batch, FEATURES, dtype=torch.bfloat16, device=x.device)
-    gf = torch.empty(batch, FEATURES, dtype=torch.float32, device=x.device) if want_f32 else None
+        grad_out = torch.empty(batch, feats, dtype=torch.bfloat16, device=x.device)
+    gf = torch.empty(batch, feats, dtype=torch.float32, device=x.device) if want_f32 else None
     sarr = None
     if seeds is not None:
         sarr = (ctypes.c_uint32 * nc)(*[int(s) & 0xFFFFFFFF for s in seeds])
     if loss_out is not None:
         assert loss_out.is_cuda and loss_out.dtype == torch.float32 and loss_out.numel() == 1
     st = lib.xmc_tiled_step_ex(arr, nc, rows_per_chunk, chunk_views[-1].shape[0], WEIGHT_TYPES[weight_type], x.data_ptr(),
-                            batch, FEATURES, labels.data_ptr() if labels.numel() else None, labels.shape[0], float(lr),
+                            batch, feats, labels.data_ptr() if labels.numel() else None, labels.shape[0], float(lr),
                             sarr, _lib.ROUND_MODES[round_mode], int(bool(quantize_x)), int(bool(saturate)),
                             kahan.data_ptr() if kahan is not None else None, ktype, int(num_head), float(weight_decay),
                             float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, grad_out.data_ptr(),

@@ -53,7 +53,9 @@ class XMCBCECHUNKEDLayer(nn.Module):
         assert self._dtype in (torch.bfloat16, torch.float32, torch.float16), f"unsupported weight type {self._dtype}"
         assert self.device.type == "cuda", "XMCBCECHUNKEDLayer needs a GPU device: there is no CPU path"
         features = cfg.model.xmc.input_features
-        assert features == ops.FEATURES, f"the gfx950 kernels are built for {ops.FEATURES} input features"
+        assert features in ops.TILED_FEATURES or self._dtype != torch.bfloat16, \
+            f"the gfx950 kernels of the bf16 layer are built for {ops.TILED_FEATURES} input features"
+        self.features = features
 
         num_labels = cfg.data.num_labels
         self.num_labels = num_labels
@@ -76,11 +78,12 @@ class XMCBCECHUNKEDLayer(nn.Module):
         self._workspace = None
         if self._dtype == torch.bfloat16:
             self._workspace = ops.alloc_tiled_workspace(self.num_chunks, self.chunk_size, self.device,
-                                                        min(max(int(cfg.data.batch_size), ops.MAX_BATCH), ops.MAX_BATCH_TILED))
+                                                        min(max(int(cfg.data.batch_size), ops.MAX_BATCH), ops.MAX_BATCH_TILED),
+                                                        features)
 
     def _chunks(self):
         w = self.xfc_weight
-        assert w.is_contiguous() and w.dtype == self._dtype and w.shape == (self.num_labels, ops.FEATURES)
+        assert w.is_contiguous() and w.dtype == self._dtype and w.shape == (self.num_labels, self.features)
         views = []
         for c in range(self.num_chunks):
             lo, hi = c * self.chunk_size, min((c + 1) * self.chunk_size, self.num_labels)
@@ -109,7 +112,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
         '''
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args:
-            embed: Encoder or bottleneck layer output, [B, 768], B <= 512 (any value; bf16 weights).
+            embed: Encoder or bottleneck layer output, [B, 768] or [B, 1024], B <= 512 (any value; bf16 weights).
             labels: Positive labels in sparse format (row,col). shape = (Nb,2).
             xmc_lr: list of learning rates, only [0] is used.
             skip_loss: Whether to skip the loss calculation.  When False the summed binary cross entropy of the step's
@@ -117,7 +120,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
                        the value the reference's _compute_loss is written to return (chunked.py:57-72); the reference
                        itself passes the weight chunk where the logits belong (chunked.py:109).
         '''
-        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
+        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == self.features
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
         if self._dtype != torch.bfloat16:
             return self._dense_step(embed.detach(), labels, xmc_lr, skip_loss)
@@ -148,7 +151,7 @@ class XMCBCECHUNKEDLayer(nn.Module):
         bsz = embed.shape[0]
         if embed.dtype != self._dtype:
             embed = embed.to(self._dtype)                                          # :89-90
-        grad_input = torch.zeros(bsz, ops.FEATURES, dtype=torch.float32, device=self.device)   # :93
+        grad_input = torch.zeros(bsz, self.features, dtype=torch.float32, device=self.device)   # :93
         for chunk_idx in range(self.num_chunks):
             start_idx = chunk_idx * self.chunk_size
             end_idx = min(start_idx + self.chunk_size, self.num_labels)

@@ -26,7 +26,7 @@ extern "C" {
 enum {
   XMC_OK = 0,
   XMC_ERR_NULL = -1,        /* a required pointer is null */
-  XMC_ERR_SHAPE = -2,       /* unsupported shape (features != 768, batch > 128 or not a multiple of 16, rows % 16 != 0, ...) */
+  XMC_ERR_SHAPE = -2,       /* unsupported shape (features != 768 - tiled path: 768 or 1024 -, batch > 128 or not a multiple of 16, rows % 16 != 0, ...) */
   XMC_ERR_ALIGN = -3,       /* a device pointer is not 16-byte aligned */
   XMC_ERR_RANGE = -4,       /* too many chunks / positives / labels for this build */
   XMC_ERR_WORKSPACE = -5,   /* workspace smaller than xmc_workspace_bytes() */
@@ -189,6 +189,9 @@ enum {
 
 /* Bytes of workspace xmc_tiled_step needs for batches of up to max_batch rows (1..512). */
 size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_batch);
+/* The same for a layer of `features` inputs (768 or 1024; the function above is this one at 768).  0 for any other
+ * width. */
+size_t xmc_tiled_workspace_bytes_ex(int num_chunks, int rows_per_chunk, int max_batch, int features);
 
 /* One training step of the modes in which the reference keeps bf16 temporaries, three kernels per chunk as there:
  *   XMC_WEIGHT_BF16  XMCBCECHUNKEDLayer.xfc_forward_backward (chunked.py:76-133) with sgd_update
@@ -197,7 +200,9 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *   XMC_WEIGHT_E4M3  Fp8XMCBCEChunkedLayer with simulated_fp8 (chunked_fp8xmc_clf.py:98-99,110,115-116;
  *                    fuse_kernel.py:184-199): logits from the un-quantised bf16 X, W = e4m3_torch(SR20(W - lr*A)),
  *                    where the final cast does not saturate (NaN above 464)
- *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, 768] row-major each; all chunks
+ *   features         768 or 1024 (d below); XMC_ERR_SHAPE otherwise.  The workspace is sized by
+ *                    xmc_tiled_workspace_bytes_ex for the same width
+ *   chunk_ptrs       host array of device pointers to the chunks' first rows; [rows, d] row-major each; all chunks
  *                    have rows_per_chunk rows except the last (rows_last_chunk <= rows_per_chunk); any row count
  *   labels_coo       as xmc_fp8_step; label id = chunk * rows_per_chunk + row.  The label space may exceed the 2^24 labels
  *                    the sort keys of xmc_fp8_step hold (up to 2^31 - 1 labels, a chunk below 2^24 - 1 rows): the
@@ -209,7 +214,7 @@ size_t xmc_tiled_workspace_bytes(int num_chunks, int rows_per_chunk, int max_bat
  *   saturate         e4m3 weights: 0 = final cast as torch (NaN above 464, :116), 1 = saturating at +-448 (fuse_kernel.py:35)
  *   kahan, kahan_type, num_head
  *                    head-Kahan update of Fp8XMCBCEChunkedHeadKahanLayer (chunked_head_kahan_fp8xmc_clf.py:41-48,127-131;
- *                    fuse_kernel.py:202-262), e4m3 weights only: device buffer [num_head, 768] of bf16 (kahan_type 1) or
+ *                    fuse_kernel.py:202-262), e4m3 weights only: device buffer [num_head, d] of bf16 (kahan_type 1) or
  *                    e5m2 (kahan_type 2) for the first num_head rows of chunk 0, updated in place; kahan_type 0 = none
  *   loss_out         device float or null.  Not null: receives the summed binary cross entropy of the step's bf16 logits
  *                    against the targets, sum over labels and batch rows of max(z,0) - [positive] z + log(1 + exp(-|z|)),

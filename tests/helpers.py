@@ -8,10 +8,10 @@ from oracle import step as O
 
 
 def make_case(num_chunks, rows_per_chunk, batch, seed, pos_mean=5.0, zipf_s=1.0, std=0.02, extra_labels=None,
-              w_scale=1.0):
+              w_scale=1.0, features=768):
     L = num_chunks * rows_per_chunk
-    x = synth.make_x(batch, 768, seed)
-    w = synth.make_weights_np(L, 768, seed, std) / np.float32(w_scale)
+    x = synth.make_x(batch, features, seed)
+    w = synth.make_weights_np(L, features, seed, std) / np.float32(w_scale)
     codes = C.e4m3_encode(w, saturate=True)
     labels = synth.make_labels(batch, L, pos_mean, zipf_s, seed)
     if extra_labels is not None:
