@@ -73,7 +73,6 @@ struct RBlockLane {
   unsigned orow_lane;    // image of updated weights: the same 12 bytes
   unsigned gcol;         // first of the lane's 12 features
   unsigned hash_lane;    // lane part of the random-word hash
-  unsigned char* dummy;  // where stores of rows past the end of a chunk go (nobody reads it)
 };
 
 // The compensation terms of one A^T block (head-Kahan layer): 12 per lane, raw (bf16: six dwords, e5m2: three), and
@@ -239,7 +238,6 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   bl.orow_lane = (unsigned)(l16 * QCOLS + 48 * f + 12 * kg);
   bl.gcol = (unsigned)(QCOLS * m + 48 * f + 12 * kg);
   bl.hash_lane = ((unsigned)l16 * (unsigned)(D / 4) + (bl.gcol >> 2)) * 0x9E3779B1u;
-  bl.dummy = exq + (size_t)(m * 2 + (v >> 2)) * QG_BYTES + RG_BYTES + f * 1024 + lane * 16;
   bf16x8 xt[3][4];       // grad_W: feature blocks of this wavefront's 48 features, K steps of 32 batch rows
 #pragma unroll
   for (int cg = 0; cg < 3; cg++)
@@ -466,6 +464,8 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     // descriptors of the next iteration: the tile of its stage A (whose columns it also fetches), the tile whose rows it
     // fetches and the tile of its share of stage B; loaded one iteration ahead through the scalar path
     QTile qa_n = q_desc_full(cdesc, tile_at(RQ)), qr_n = q_desc_head(cdesc, tile_at(RQ + RR_RING - 1)), qb_n = q_desc_full(cdesc, tile_at(0));
+    unsigned char* qp_base = nullptr;   // the tile of the iteration before: base pointer and valid rows
+    int qp_base_valid = 0;
     int sa = RQ % RR_RING;    // (i + RQ) % RR_RING, the rows image stage A reads
     int w0 = 0;               // i % RC_RING
     for (int i = 0; i < n_it; i++) {
@@ -517,6 +517,25 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       qr_n = q_desc_head(cdesc, tile_at(i + 1 + RQ + RR_RING - 1));
       qb_n = q_desc_full(cdesc, tile_at(i + 1));
       if (do_a) stage_a_finish(i + RQ, qa, z);
+      // the previous tile's updated weights, from their LDS image to memory: 12 wave-wide pieces of 16 bytes per lane,
+      // three per A wavefront (chunk ch = (3a + jj) * 64 + lane is bytes 16 (ch % 12).. of row ch / 12)
+      if (i > 0) {
+#pragma unroll
+        for (int jj = 0; jj < 3; jj++) {
+          const int ch = (3 * a + jj) * 64 + lane, row = ch / 12;
+          const unsigned off = (unsigned)(row * D + QCOLS * m + (ch - row * 12) * 16);
+          const intx4 ov = *(const __attribute__((address_space(3))) intx4*)(lds + RLDS_O + ((i + 1) & 1) * RO_BYTES + ch * 16);
+          if (qp_base_valid == TL) {
+            asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(off), "v"(ov), "s"(qp_base) : "memory");
+          } else {
+            // rows past the end of the chunk go to a place nobody reads (the padding behind an exchange slot), so that
+            // the wavefront issues the same number of memory operations for every tile
+            unsigned char* dst = row < qp_base_valid ? qp_base + off : exq + (size_t)(m * 2) * QG_BYTES + RG_BYTES + a * 1024 + lane * 16;
+            asm volatile("global_store_dwordx4 %0, %1, off ; clamped rows" : : "v"(dst), "v"(ov) : "memory");
+          }
+        }
+      }
+      qp_base = qb.base; qp_base_valid = qb.rows_valid;
       // ---- the update of those blocks, with the rows of position i + RQ + 2 (the only loads that miss the L2) requested
       //      between its pieces
       {
@@ -539,12 +558,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       // Loads and stores complete in order.  Waiting for all but the stores of G and the rows covers the gather, the
       // columns and the snapshot, all issued long before, and everything of the iteration before, whose stores of G can
       // now be published.
-      if (do_a) {
-        if (ra == 0) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-      } else {
-        if (ra == 0) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+      {
+        const int cnt = (do_a ? 2 : 0) + (i > 0 ? 3 : 0) + (ra == 0 ? 4 : 3);
+        switch (cnt) {
+          case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+          case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+          case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+          case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+          case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+          case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+          default: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+        }
       }
       if (lane == 0) __hip_atomic_store(myflag, min(i + RQ, n_it), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       sa = sa == RR_RING - 1 ? 0 : sa + 1;
@@ -580,35 +604,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     if (k + 1 < RQ && k + 1 >= RR_RING) __syncthreads();
   }
 
-  // The image of a tile's updated weights (64 rows x 192 bytes) goes to memory as 12 wave-wide stores of 16 bytes per
-  // lane, three per B wavefront: chunk ch = (3s + j) * 64 + lane is bytes 16 (ch % 12).. of row ch / 12.
-  unsigned so_lds[3], so_mem[3];
-  int so_row[3];
-#pragma unroll
-  for (int jj = 0; jj < 3; jj++) {
-    const int ch = (3 * s + jj) * 64 + lane;
-    so_row[jj] = ch / 12;
-    so_lds[jj] = (unsigned)(ch * 16);
-    so_mem[jj] = (unsigned)(so_row[jj] * D + QCOLS * m + (ch - so_row[jj] * 12) * 16);
-  }
-  auto so_read = [&](int slot, int jj) { return *(const __attribute__((address_space(3))) intx4*)(lds + RLDS_O + slot * RO_BYTES + so_lds[jj]); };
-  auto so_store = [&](const QTile& qp, int jj, const intx4& ov) {
-    typedef __attribute__((address_space(1))) intx4 gi4;
-    unsigned char* dst = so_row[jj] < qp.rows_valid ? qp.base + so_mem[jj] : bl.dummy;
-    // plain stores on purpose: non-temporal ones keep the exchanged G tiles and the tiles between their two fetches in
-    // the XCD's L2 (reads from memory drop from 1.34 to 1.05 times the weights) but cost 5 % of the kernel's time
-    *(gi4*)(unsigned long long)dst = ov;
-  };
-  auto store_out = [&](const QTile& qp, int slot) {
-    intx4 ov[3];
-#pragma unroll
-    for (int jj = 0; jj < 3; jj++) ov[jj] = so_read(slot, jj);
-#pragma unroll
-    for (int jj = 0; jj < 3; jj++) so_store(qp, jj, ov[jj]);
-  };
-
   QTile q_n = q_desc_full(cdesc, tile_at(0)), q_p = q_n;
-  q_p.rows_valid = 0;   // no previous tile yet: the first iteration's stores all go to the dummy place
   int w0 = 0;   // i % RC_RING
   int n_done = 0;
   for (int i = 0; i < n_it; i++) {
@@ -660,15 +656,12 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     unsigned wq[2][3];      // their old weights
     float t[3][4];
     unsigned hs[3], outw[3];
-    intx4 so_v;   // a piece of the previous tile's updated weights on its way from LDS to memory
     RKahanBlock kb[2] = {};   // compensation terms of the block in progress and of the one being rounded
     // (this loop must be unrolled completely: its register arrays are indexed by k.  The variants with the Philox
     // recipe or a compensated head exceed the compiler's default size limit for "#pragma unroll" and are compiled in a
     // translation unit of their own, xmc_fp8_role_heavy.hip, with a higher limit.)
 #pragma unroll
     for (int k = 0; k < NS; k++) {
-      if ((k & 7) == 1 && k < 24) so_v = so_read((i + 1) & 1, k >> 3);
-      if ((k & 7) == 5 && k < 24) so_store(q_p, k >> 3, so_v);
       request(k + PD);
       // vector pieces of this step
       if (k == 0) {
@@ -738,7 +731,17 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __syncthreads();   // every wavefront has written its part of the last tile's image
-  if (n_done > 0) store_out(q_p, (n_done + 1) & 1);
+  // The image of the last tile's updated weights (64 rows x 192 bytes) goes to memory as 12 wave-wide stores of 16 bytes
+  // per lane, three per B wavefront (the A wavefronts, which store the other tiles' images one iteration later, have
+  // left): chunk ch = (3s + jj) * 64 + lane is bytes 16 (ch % 12).. of row ch / 12.
+  if (n_done > 0) {
+#pragma unroll
+    for (int jj = 0; jj < 3; jj++) {
+      const int ch = (3 * s + jj) * 64 + lane, row = ch / 12;
+      const intx4 ov = *(const __attribute__((address_space(3))) intx4*)(lds + RLDS_O + ((n_done + 1) & 1) * RO_BYTES + ch * 16);
+      if (row < q_p.rows_valid) *(intx4*)(q_p.base + (size_t)(row * D + QCOLS * m + (ch - row * 12) * 16)) = ov;
+    }
+  }
 
   // ---- per-workgroup grad_X partial, summed in a fixed order by reduce_gx_role_kernel: [24 blocks][4 B wavefronts][64 lanes]
   floatx4* dst = p.partial + (size_t)g * 24 * 256;
