@@ -56,8 +56,13 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self.num_labels_i = self.num_labels // self.num_chunks
         assert self.num_labels_i % 16 == 0
         features = cfg.model.xmc.input_features
-        assert features == ops.FEATURES, f"the gfx950 kernels are built for {ops.FEATURES} input features"
+        assert features in ops.TILED_FEATURES, f"the gfx950 kernels are built for {ops.TILED_FEATURES} input features"
         assert self.device.type == "cuda", "Fp8XMCBCEChunkedLayer needs a GPU device: there is no CPU path"
+        self.features = features
+        # The fused step and the inference kernels are built for 768 features.  A layer of 1,024 trains on the
+        # three-kernel path (same arithmetic, rounding modes and random words) and takes its inference logits from a
+        # library GEMM per chunk on the exactly widened operands, as the reference does (:52-55).
+        self._other_width = features != ops.FEATURES
 
         # same initialisation as the reference (:29-32): xavier-uniform on the padded fp32 matrix, cast per chunk
         xfc_weight = torch.empty(self.num_labels, features, dtype=torch.float32)
@@ -86,7 +91,8 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         self.iteration = 0
         self.grad_input = None
         # all scratch memory of the step comes from the torch allocator (so that max_memory_allocated sees it)
-        self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
+        self._workspace = (None if self._other_width else
+                           ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device))
         self._tiled_workspace = None
         self._fused_ran = False      # the error word in the workspace is defined once a fused step has run
         # After every fused step the workspace's sticky error word (the error words of all steps since it was last
@@ -94,7 +100,7 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         # later calls look at the copies that have arrived (see _check_previous_steps).  A ring of slots, so that a copy
         # still in flight is never overwritten by the next one.
         off = ops.step_sticky_error_offset()
-        self._err_dev = self._workspace[off:off + 4].view(torch.int32)
+        self._err_dev = None if self._other_width else self._workspace[off:off + 4].view(torch.int32)
         self._err_slots = 4
         self._err_host = torch.zeros(self._err_slots, dtype=torch.int32).pin_memory()
         self._err_events = [None] * self._err_slots
@@ -106,9 +112,12 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         # the fused kernel's sort keys hold 24 bits of label: larger label spaces run on the three-kernel path, which sorts
         # the positives per segment of the label space
         self._wide = self.num_labels >= (1 << 24) - 1
-        if self.fake_fp8_matmul or self._max_batch > ops.MAX_BATCH or self._wide:
+        if self._other_width:
+            assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales belong to the fused step (768 features)"
+        if self.fake_fp8_matmul or self._max_batch > ops.MAX_BATCH or self._wide or self._other_width:
             self._tiled_workspace = ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device,
-                                                              min(max(self._max_batch, ops.MAX_BATCH), ops.MAX_BATCH_TILED))
+                                                              min(max(self._max_batch, ops.MAX_BATCH), ops.MAX_BATCH_TILED),
+                                                              features)
 
     def _chunks(self):
         return [w.data for w in self.xfc_weight]
@@ -122,6 +131,14 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         outs = [torch.matmul(x, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
         return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
 
+    def _widened_logits(self, embed):
+        # true-FP8 logits (:53-56) for a width the inference kernel is not built for: Z = W_i e4m3(X)^T per chunk through
+        # the library's bf16 GEMM.  Both operands are e4m3 values, which bf16 holds exactly, and the products are summed
+        # in fp32, so only the order of the fp32 sums differs from an FP8 GEMM.
+        xq = embed.to(torch.float8_e4m3fn).to(torch.bfloat16)
+        outs = [torch.matmul(xq, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
+        return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
+
     @torch.no_grad()
     def xfc_forward(self, embed):
         '''
@@ -130,6 +147,8 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         assert embed.is_cuda and embed.dim() == 2
         if self.fake_fp8_matmul:
             return self._simulated_logits(embed)
+        if self._other_width:
+            return self._widened_logits(embed)
         return ops.fp8_forward(self._chunks(), embed, self.cfg.data.num_labels, self.scale_w, self.scale_x,
                                self._workspace)
 
@@ -140,8 +159,8 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         [B, num_labels] logits: the top-k is merged chunk by chunk.  Not in the reference; k <= 128.
         '''
         assert embed.is_cuda and embed.dim() == 2
-        if self.fake_fp8_matmul:
-            vals, idx = self._simulated_logits(embed).topk(k)
+        if self.fake_fp8_matmul or self._other_width:
+            vals, idx = (self._simulated_logits(embed) if self.fake_fp8_matmul else self._widened_logits(embed)).topk(k)
             return vals, idx
         return ops.fp8_forward_topk(self._chunks(), embed, self.cfg.data.num_labels, k, self.scale_w, self.scale_x,
                                     self._workspace)
@@ -161,13 +180,13 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         '''
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args:
-            embed: Encoder or bottleneck layer output, bf16 [B, 768], B a multiple of 16 and <= 512 (the fused
-                   kernel takes up to 128 rows, larger batches run on the three-kernel path).
+            embed: Encoder or bottleneck layer output, bf16 [B, 768] or [B, 1024], B a multiple of 16 and <= 512 (the
+                   fused kernel takes up to 128 rows of 768 features, everything else runs on the three-kernel path).
             labels: Positive labels in sparse format, int32 [Nb, 2] = (row in batch, label id).
             xmc_lr: list of learning rates, only [0] is used.
             skip_loss: ignored, as in the reference's FP8 layer; the return value is 0.
         '''
-        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
+        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == self.features
         assert embed.shape[0] <= ops.MAX_BATCH_TILED and (self.fake_fp8_matmul or embed.shape[0] % 16 == 0), \
             "batch must be a multiple of 16 and at most 512 (the reference data loader uses drop_last)"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
@@ -186,10 +205,10 @@ class Fp8XMCBCEChunkedLayer(nn.Module):
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, **extra)
-        elif embed.shape[0] > ops.MAX_BATCH or self._wide:
+        elif embed.shape[0] > ops.MAX_BATCH or self._wide or self._other_width:
             # the fused kernel holds 128 batch rows; larger batches take the three-kernel path with the same arithmetic
             # (logits from e4m3(X), saturating cast) and the same rounding modes and random words
-            assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128"
+            assert self.scale_w == 1.0 and self.scale_x == 1.0, "per-tensor scales need a batch of at most 128 rows of 768 features"
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
                                              saturate=True, **extra)

@@ -41,7 +41,11 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
         self.num_labels_i = self.num_labels // self.num_chunks
         assert self.num_labels_i % 16 == 0
         features = cfg.model.xmc.input_features
-        assert features == ops.FEATURES, f"the gfx950 kernels are built for {ops.FEATURES} input features"
+        assert features in ops.TILED_FEATURES, f"the gfx950 kernels are built for {ops.TILED_FEATURES} input features"
+        self.features = features
+        # 768 features: fused step and inference kernel; 1,024: three-kernel path (same arithmetic) and a library GEMM per
+        # chunk on the exactly widened operands for inference, as the reference does (:64-67)
+        self._other_width = features != ops.FEATURES
         assert self.device.type == "cuda", "Fp8XMCBCEChunkedHeadKahanLayer needs a GPU device: there is no CPU path"
 
         xfc_weight = torch.empty(self.num_labels, features, dtype=torch.float32)
@@ -63,16 +67,16 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
             kdt = torch.float8_e5m2 if self.fp8_head_kahan else torch.bfloat16
             self.head_kahan = torch.zeros(self.num_head, features, dtype=kdt, device=self.device)
             assert 0 < self.num_head <= self.num_labels_i
-        self._tiled = bool(self.fake_fp8_matmul or self.using_head_kahan)
+        self._tiled = bool(self.fake_fp8_matmul or self.using_head_kahan or self._other_width)
         self.rounding = _opt(cfg.training.xmc, "rounding", "sr_philox" if self.fake_fp8_matmul else "sr_fast")
         assert self.rounding in (("sr_philox", "rtn") if self.fake_fp8_matmul else ("sr_fast", "sr_philox", "rtn"))
         self.block_size = 16
         self.loss = torch.tensor(0.0, device=self.device)
         self.iteration = 0
         self.grad_input = None
-        self._workspace = ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
-        self._tiled_workspace = (ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device)
-                                 if self._tiled else None)
+        self._workspace = None if self._other_width else ops.alloc_workspace(self.num_chunks, self.num_labels_i, self.device)
+        self._tiled_workspace = (ops.alloc_tiled_workspace(self.num_chunks, self.num_labels_i, self.device, ops.MAX_BATCH,
+                                                           features) if self._tiled else None)
 
     def _chunks(self):
         return [w.data for w in self.xfc_weight]
@@ -88,6 +92,11 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
             x = embed.to(torch.bfloat16)
             outs = [torch.matmul(x, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
             return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
+        if self._other_width:
+            # e4m3 operands widened exactly to bf16, fp32 sums: only their order differs from an FP8 GEMM
+            xq = embed.to(torch.float8_e4m3fn).to(torch.bfloat16)
+            outs = [torch.matmul(xq, w.data.to(torch.bfloat16).t()) for w in self.xfc_weight]
+            return torch.cat(outs, dim=1)[:, :self.cfg.data.num_labels]
         return ops.fp8_forward(self._chunks(), embed, self.cfg.data.num_labels, 1.0, 1.0, self._workspace)
 
     @torch.no_grad()
@@ -102,7 +111,7 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
         Computes activation gradients for the XMC layer fused with BCE Loss and applies the SGD update.
         Args as Fp8XMCBCEChunkedLayer.xfc_forward_backward; skip_loss is ignored as in the reference; returns 0.
         '''
-        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == ops.FEATURES
+        assert embed.is_cuda and embed.dim() == 2 and embed.shape[1] == self.features
         assert embed.shape[0] <= ops.MAX_BATCH and (self._tiled or embed.shape[0] % 16 == 0), \
             "batch must be a multiple of 16 and at most 128 (the reference data loader uses drop_last)"
         assert labels.is_cuda and labels.dim() == 2 and labels.shape[1] == 2
@@ -117,13 +126,17 @@ class Fp8XMCBCEChunkedHeadKahanLayer(nn.Module):
         if self.fake_fp8_matmul:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace)
-        elif self.using_head_kahan and embed.shape[0] % 16 == 0:
+        elif self.using_head_kahan and embed.shape[0] % 16 == 0 and not self._other_width:
             self.grad_input = ops.fp8_kahan_step(self._chunks(), self.head_kahan, self.num_head, x, lab, xmc_lr[0],
                                                  seeds=seeds, round_mode=self.rounding, workspace=self._workspace)
         elif self.using_head_kahan:
             self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
                                              round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
                                              saturate=True, kahan=self.head_kahan, num_head=self.num_head)
+        elif self._other_width:
+            self.grad_input = ops.tiled_step(self._chunks(), self.num_labels_i, "e4m3", x, lab, xmc_lr[0], seeds=seeds,
+                                             round_mode=self.rounding, workspace=self._tiled_workspace, quantize_x=True,
+                                             saturate=True)
         else:
             self.grad_input = ops.fp8_step(self._chunks(), x, lab, xmc_lr[0], seeds=seeds, round_mode=self.rounding,
                                            workspace=self._workspace)

@@ -209,3 +209,61 @@ def test_chunked_module_at_1024(gpu):
         w = xfc.xfc_weight.float().cpu().numpy()
     logits = xfc.xfc_forward(emb)
     assert logits.shape == (48, 3000)
+
+
+def test_fp8_modules_at_1024(gpu):
+    """Fp8XMCBCEChunkedLayer and the head-Kahan layer with input_features = 1024: the step runs on the three-kernel path
+    with the true-FP8 arithmetic (oracle: fp8_step / fp8_kahan_step), inference through a library GEMM per chunk on the
+    exactly widened operands (oracle: fp8_forward, whose products are the same and whose fp32 sums differ in order)."""
+    import types
+    import torch
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked_fp8xmc_clf import Fp8XMCBCEChunkedLayer
+    from xmc_classifiers.chunked_head_kahan_fp8xmc_clf import Fp8XMCBCEChunkedHeadKahanLayer
+    cfg = make_cfg("cuda:0", 2000, 2, rounding="rtn")
+    cfg.model.xmc.input_features = FEATS
+    torch.manual_seed(7)
+    xfc = Fp8XMCBCEChunkedLayer(cfg)
+    assert [tuple(w.shape) for w in xfc.xfc_weight] == [(1008, FEATS)] * 2 and xfc._dtype == torch.float8_e4m3fn
+    x = synth.make_x(48, FEATS, 201)
+    labels = synth.make_labels(48, 2000, 5.0, 1.0, 201).astype(np.int32)
+    emb = torch.from_numpy(C.bf16_bits(x).view(np.int16)).to(gpu).view(torch.bfloat16)
+    w0 = [w.data.view(torch.uint8).cpu().numpy().copy() for w in xfc.xfc_weight]
+    assert xfc.xfc_forward_backward(emb, torch.from_numpy(labels).to(gpu), [0.05]) == 0 and xfc.iteration == 1
+    ref_codes, ref_gx, ref_gi = O.fp8_step(w0, x, labels, 0.05, sr_mode="rtn")
+    assert code_mismatch([w.data.view(torch.uint8).cpu().numpy() for w in xfc.xfc_weight], ref_codes) < 2e-3
+    assert xfc.grad_input.shape == (48, FEATS) and xfc.grad_input.dtype == torch.bfloat16
+    H.assert_bf16_close(xfc.grad_input.float().cpu().numpy(), ref_gi)
+    assert xfc.last_step_error() == 0
+    xfc.check_steps()
+    # inference: as the evaluator calls it (embedding cast to the layer's type first), dense and top-k
+    w1 = [w.data.view(torch.uint8).cpu().numpy() for w in xfc.xfc_weight]
+    logits = xfc.xfc_forward(emb.to(xfc._dtype))
+    ref = O.fp8_forward(w1, x, 2000)
+    assert logits.shape == (48, 2000) and logits.dtype == torch.bfloat16
+    H.assert_bf16_close(logits.float().cpu().numpy(), ref)
+    vals, idx = xfc.xfc_forward_topk(emb.to(xfc._dtype), 10)
+    tv, ti = logits.topk(10)
+    assert torch.equal(vals, tv) and torch.equal(idx, ti)
+    # the default rounding of this width is the fast stochastic one, on the same path
+    cfg_sr = make_cfg("cuda:0", 2000, 2)
+    cfg_sr.model.xmc.input_features = FEATS
+    xfc_sr = Fp8XMCBCEChunkedLayer(cfg_sr)
+    assert xfc_sr.rounding == "sr_fast" and xfc_sr.xfc_forward_backward(emb, torch.from_numpy(labels).to(gpu), [0.05]) == 0
+
+    # head-Kahan layer
+    cfgk = make_cfg("cuda:0", 1000, 2, rounding="rtn")
+    cfgk.model.xmc.input_features = FEATS
+    cfgk.training.FP8 = types.SimpleNamespace(using_head_kahan=True, fp8_head_kahan=False, head_ratio=0.2)
+    torch.manual_seed(8)
+    xk = Fp8XMCBCEChunkedHeadKahanLayer(cfgk)
+    assert xk.num_labels == 1024 and xk.num_head == 204 and xk.head_kahan.shape == (204, FEATS)
+    tokens = emb[:32]
+    lab = torch.tensor([[0, 3], [31, 999], [4, 100]], dtype=torch.int32, device=gpu)
+    before = [w.view(torch.uint8).cpu().numpy().copy() for w in xk.xfc_weight]
+    assert xk.xfc_forward_backward(tokens, lab, [0.05]) == 0
+    ref_codes, ref_k, _, _ = O.fp8_kahan_step(before, np.zeros((204, FEATS), np.float32), x[:32], lab.cpu().numpy(), 0.05, 204,
+                                              sr_mode="rtn")
+    assert code_mismatch([w.view(torch.uint8).cpu().numpy() for w in xk.xfc_weight], ref_codes) < 2e-3
+    assert float(xk.head_kahan.float().abs().max()) > 0
+    assert xk.xfc_forward(tokens.to(xk._dtype)).shape == (32, 1000)
