@@ -62,6 +62,8 @@ def load():
     lib.xmc_step_error_word.argtypes = [vp, i32, i32, vp]
     lib.xmc_tiled_workspace_bytes.restype = sz
     lib.xmc_tiled_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.xmc_debug_spin_limit.restype = i32
+    lib.xmc_debug_spin_limit.argtypes = [i32]
     lib.xmc_tiled_workspace_bytes_ex.restype = sz
     lib.xmc_tiled_workspace_bytes_ex.argtypes = [i32, i32, i32, i32]
     lib.xmc_tiled_step.restype = i32

@@ -8,6 +8,7 @@
 #include "xmc_topk.hip"
 #include "xmc_dropout.hip"
 #include <stdlib.h>
+#include <atomic>
 #include <mutex>
 
 using namespace xmc;
@@ -80,6 +81,9 @@ DeviceInfo device_info() {
   std::call_once(g_device_once[dev], fill_device_info, dev);
   return g_device_info[dev];
 }
+
+// polls of a partner's counter before a workgroup of the fused step gives up (xmc_debug_spin_limit)
+std::atomic<int> g_spin_limit{QSPIN_LIMIT};
 
 // optional event pair recorded around the next launch of the fused step kernel by the calling thread (benchmarking aid)
 thread_local hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;
@@ -267,6 +271,7 @@ static int fused_step(void* const* chunk_ptrs, int num_chunks, int rows_per_chun
     p.kmax = (rest_tiles + p.nquads - 1) / p.nquads;
     p.cnt_base = 0;
     p.acc_init = 0;
+    p.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     quad_sort_kernel<<<n_pad > 0 ? n_pad / 64 : 1, 256, (size_t)(n_pad + 256) * 4, stream>>>(
         labels_coo, nnz, n_pad, batch, 0, 0, num_chunks * rows_per_chunk, (unsigned*)(ws + WS_KEYS), (int*)(ws + WS_FLAGS));
     const int desc_blocks = (num_tiles + 1 + 255) / 256;
@@ -526,6 +531,10 @@ int xmc_dropout_quantize(const void* x, int x_type, int rows, int cols, float p,
   dropout_quantize_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, (hipStream_t)stream_>>>(x, x_type, n4, cols, p, (unsigned)(seed & 0xFFFFFFFFull),
                                                                                         (unsigned)(seed >> 32), (unsigned*)out_e4m3);
   return launch_status();
+}
+
+int xmc_debug_spin_limit(int limit) {
+  return g_spin_limit.exchange(limit < 0 ? QSPIN_LIMIT : limit, std::memory_order_relaxed);
 }
 
 int xmc_profile_events(void* start_event, void* stop_event) {

@@ -57,6 +57,8 @@ struct QuadParams {
   int num_head, head_tiles, kmax_head;
   int cnt_base;                       // first of this launch's tiles-published counters in flags
   int acc_init;                       // the grad_X partials continue from what the launch before left in `partial`
+  int spin_limit;                     // polls of a partner's counter before a workgroup gives up (QSPIN_LIMIT; a test aid
+                                      // lowers it to exercise the give-up path)
 };
 
 #define QFENCE() __builtin_amdgcn_sched_barrier(0)   // nothing is scheduled across this point

@@ -321,7 +321,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       for (int spin = 0;; spin++) {
         int fl = __hip_atomic_load(srcflags + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__builtin_amdgcn_read_exec() == __builtin_amdgcn_ballot_w64(fl >= need)) break;
-        if (spin >= QSPIN_LIMIT || ((spin & 1023) == 1023 && __hip_atomic_load(errw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+        if (spin >= p.spin_limit || ((spin & 1023) == 1023 && __hip_atomic_load(errw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
           // give up: raise the error word (partners that wait for this workgroup see it and give up too) and the
           // workgroup's abort word; every wavefront leaves the loop behind the next barrier
           if (lane == 0) {

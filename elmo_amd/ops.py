@@ -312,6 +312,12 @@ def tiled_step(chunk_views, rows_per_chunk, weight_type, x, labels, lr, seeds=No
     return (grad_out, gf) if want_f32 else grad_out
 
 
+def debug_spin_limit(limit):
+    """Test aid: polls of a partner's counter before a workgroup of the fused step gives up (negative: the default);
+    returns the previous value."""
+    return int(_lib.load().xmc_debug_spin_limit(int(limit)))
+
+
 def step_error_offset():
     """Byte offset of the fused step's error word (int32) inside its workspace."""
     return int(_lib.load().xmc_step_error_offset())

@@ -176,6 +176,13 @@ int xmc_fp8_forward_topk_fused(void* const* chunk_ptrs, int num_chunks, int rows
 int xmc_dropout_quantize(const void* x, int x_type, int rows, int cols, float p, unsigned long long seed, void* out_e4m3,
                          void* stream);
 
+/* Test aid (no counterpart in the reference): sets how often a workgroup of the fused step polls a partner's counter
+ * before it gives up (see xmc_fp8_step), for all later calls of the process, and returns the previous value; a negative
+ * `limit` restores the default (2^18 polls).  With a limit of 0 every wait that is not satisfied at once expires: the
+ * step then ends early with bit 0 of its error word set, every kernel still exits normally, and the tiles it did not
+ * reach keep their old weights.  The tests use it to exercise the give-up path. */
+int xmc_debug_spin_limit(int limit);
+
 /* Benchmarking aid (no counterpart in the reference): the next xmc_fp8_step call records these two HIP events
  * (hipEvent_t, created by the caller) immediately before and after its fused step kernel, on the call's stream,
  * then forgets them.  Pass nulls to cancel. */

@@ -21,7 +21,7 @@ def test_every_declared_symbol_is_exported():
     lib = _lib.load()
     names = declared_functions()
     assert {"xmc_version", "xmc_error_string", "xmc_workspace_bytes", "xmc_fp8_step", "xmc_fp8_forward",
-            "xmc_step_error_word", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_sticky_error_offset", "xmc_fp8_step_ex", "xmc_fp8_kahan_step", "xmc_tiled_step_ex", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_tiled_workspace_bytes_ex", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes", "xmc_fp8_forward_topk_fused", "xmc_topk_fused_scratch_bytes", "xmc_dropout_quantize"} <= set(names)
+            "xmc_step_error_word", "xmc_debug_spin_limit", "xmc_profile_events", "xmc_copy_probe", "xmc_step_error_offset", "xmc_step_sticky_error_offset", "xmc_fp8_step_ex", "xmc_fp8_kahan_step", "xmc_tiled_step_ex", "xmc_step_workgroups", "xmc_step_xcc_ids", "xmc_quad_placement_check", "xmc_fp8_forward_static", "xmc_tiled_step", "xmc_tiled_workspace_bytes", "xmc_tiled_workspace_bytes_ex", "xmc_fp8_forward_topk", "xmc_topk_scratch_bytes", "xmc_fp8_forward_topk_fused", "xmc_topk_fused_scratch_bytes", "xmc_dropout_quantize"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 

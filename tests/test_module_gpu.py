@@ -248,3 +248,75 @@ def test_step_kernels_keep_the_sticky_error_word(gpu):
     ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws)
     ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws)
     assert int(sticky.item()) == 4 and ops.step_error_word(ws, 1, 64) == 0
+
+
+def test_give_up_path_of_the_fused_step(gpu):
+    """The bounded waits of the fused step, forced to expire from the host (a polling limit of 0: a wait that is not
+    satisfied at once gives up).  Every kernel must still exit normally; the step's error word and the sticky word
+    carry bit 0; and no weight may be updated from missing data: a member's quarter of a row either keeps its old codes or
+    holds the oracle's update, because a workgroup that gives up finishes the tile whose G is complete and stops before the next.
+    The next step with the default limit is clean again, and the module turns the sticky word into an exception."""
+    import torch
+    from elmo_amd import ops
+    from test_host_cpu import make_cfg
+    from xmc_classifiers.chunked_fp8xmc_clf import Fp8XMCBCEChunkedLayer
+    nc, rows, batch = 3, 16384, 64            # 768 tiles: twelve per quad, enough for the members to drift apart
+    case = H.make_case(nc, rows, batch, 301)
+    chunks, x, labels = H.to_device_case(case, gpu)
+    ws = ops.alloc_workspace(nc, rows, gpu)
+    soff = ops.step_sticky_error_offset()
+    sticky = ws[soff:soff + 4].view(torch.int32)
+    ref_codes, _, _ = O.fp8_step(case["chunks"], case["x"], case["labels"], 0.05, sr_mode="rtn")
+    prev = ops.debug_spin_limit(0)
+    try:
+        gave_up = False
+        for attempt in range(8):              # whether a wait finds its counter at once depends on timing
+            for c, old in zip(chunks, case["chunks"]):
+                c.view(torch.uint8).copy_(torch.from_numpy(old))
+            ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws)
+            torch.cuda.synchronize()          # the kernels ran to their end
+            word = ops.step_error_word(ws, nc, rows)
+            assert word in (0, 1)
+            new = H.chunks_to_numpy(chunks)
+            updated = total = 0
+            for a, old, ref in zip(new, case["chunks"], ref_codes):
+                # the unit of the update is a member's feature quarter of a row (the members of a quad stop at
+                # different tiles)
+                same_old = (a == old).reshape(-1, 4, 192).all(axis=2)
+                good = (H.e4m3_ulp_distance(a, ref) <= 1).reshape(-1, 4, 192).all(axis=2)
+                assert np.all(same_old | good), "a row segment was updated from incomplete data"
+                updated += int((~same_old).sum()); total += same_old.size
+            if word == 1:
+                gave_up = True
+                assert int(sticky.item()) & 1
+                assert updated < total        # the step stopped early
+                break
+        assert gave_up, "no wait expired in eight steps with a polling limit of 0"
+    finally:
+        assert ops.debug_spin_limit(prev) == 0
+    # the default limit again: a clean, complete step; the sticky word keeps the earlier failure until the caller clears it
+    for c, old in zip(chunks, case["chunks"]):
+        c.view(torch.uint8).copy_(torch.from_numpy(old))
+    ops.fp8_step(chunks, x, labels, 0.05, round_mode="rtn", workspace=ws)
+    assert ops.step_error_word(ws, nc, rows) == 0 and int(sticky.item()) & 1
+    for a, ref in zip(H.chunks_to_numpy(chunks), ref_codes):
+        assert H.e4m3_ulp_distance(a, ref).max() <= 1
+    # the module raises for such a step
+    cfg = make_cfg("cuda:0", 3 * 16384 - 48, 3, rounding="rtn")
+    cfg.data.batch_size = batch
+    xfc = Fp8XMCBCEChunkedLayer(cfg)
+    prev = ops.debug_spin_limit(0)
+    try:
+        raised = False
+        for attempt in range(8):
+            try:
+                xfc.xfc_forward_backward(x, labels, [0.05])
+                xfc.check_steps()
+            except RuntimeError as e:
+                raised = "gave up waiting" in str(e)
+                break
+        assert raised
+    finally:
+        ops.debug_spin_limit(prev)
+    xfc.xfc_forward_backward(x, labels, [0.05])
+    xfc.check_steps()
