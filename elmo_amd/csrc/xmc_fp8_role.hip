@@ -92,7 +92,7 @@ struct RKahanBlock { unsigned raw[6]; bool head; int row; };
 // and on the other rows of the tile (behind the head's end) the plain update, whose random offsets count from that end.
 template <int MODE, bool WD, int KT>
 __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab)[3], const unsigned (&wq)[3], float (&t)[3][4],
-                                               unsigned (&hs)[3], unsigned (&outw)[3], const RBlockLane& bl, const QTile& q,
+                                               unsigned (&hs)[3], unsigned (&outw)[3], unsigned (&knew)[6], const RBlockLane& bl, const QTile& q,
                                                unsigned hash_tile, float lr_eff, float wd_eff, int l16, qlds_u8* lds, unsigned oimg,
                                                const RKahanBlock& kb, unsigned char* kahan, int num_head) {
   // W + k of column group cg (exact decode of both; k = 0 on rows without a term)
@@ -176,19 +176,31 @@ __device__ __forceinline__ void r_update_piece(int c, int nb, const floatx4 (&ab
         floatx2 n01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)outw[cg], false), n23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)outw[cg], true);
         kn[0] = __builtin_fmaf(-lr_eff, ab[cg][0], s[0] - n01.x); kn[1] = __builtin_fmaf(-lr_eff, ab[cg][1], s[1] - n01.y);
         kn[2] = __builtin_fmaf(-lr_eff, ab[cg][2], s[2] - n23.x); kn[3] = __builtin_fmaf(-lr_eff, ab[cg][3], s[3] - n23.y);
-        // this column group's new terms straight to memory (8 or 4 bytes per lane; the buffer is touched once per step)
-        if (kb.head) {
-          if (KT == 1) {
-            *(uint2*)(kahan + ((size_t)kb.row * D + bl.gcol + 4 * cg) * 2) = uint2{bf16_pack2(kn[0], kn[1]), bf16_pack2(kn[2], kn[3])};
-          } else {
+        // this column group's new terms, packed; the block's 24 (bf16) or 12 (e5m2) bytes per lane go to memory together
+        // behind the last column group (two stores or one instead of three: the buffer's rows are 1,536 or 768 bytes
+        // apart, and what a scattered store costs is its cache lines, not its bytes)
+        if (KT == 1) {
+          knew[2 * cg] = bf16_pack2(kn[0], kn[1]); knew[2 * cg + 1] = bf16_pack2(kn[2], kn[3]);
+        } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
-            int pk = 0;
-            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
-            pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
-            *(unsigned*)(kahan + (size_t)kb.row * D + bl.gcol + 4 * cg) = (unsigned)pk;
-          }
+          for (int e = 0; e < 4; e++) kn[e] = __builtin_fminf(__builtin_fmaxf(kn[e], -57344.0f), 57344.0f);
+          int pk = 0;
+          pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[0], kn[1], pk, false);
+          pk = __builtin_amdgcn_cvt_pk_bf8_f32(kn[2], kn[3], pk, true);
+          knew[cg] = (unsigned)pk;
         }
+      }
+    }
+    if (KT != 0 && c == 7 && kb.head) {
+      // (the lane's 24 or 12 bytes start at a multiple of 8 or 4 bytes: the vector types carry that alignment)
+      typedef unsigned k_ux4 __attribute__((ext_vector_type(4), aligned(8)));
+      typedef unsigned k_ux3 __attribute__((ext_vector_type(3), aligned(4)));
+      if (KT == 1) {
+        unsigned char* dst = kahan + ((size_t)kb.row * D + bl.gcol) * 2;
+        *(k_ux4*)dst = k_ux4{knew[0], knew[1], knew[2], knew[3]};
+        *(uint2*)(dst + 16) = uint2{knew[4], knew[5]};
+      } else {
+        *(k_ux3*)(kahan + (size_t)kb.row * D + bl.gcol) = k_ux3{knew[0], knew[1], knew[2]};
       }
     }
     if (c == 7) {
@@ -546,7 +558,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       //      between its pieces
       {
         float t[3][4];
-        unsigned hs[3], outw[3];
+        unsigned hs[3], outw[3], knew[6];
         const RKahanBlock nok = {};
         const unsigned hash_tile = qb.label0 * (unsigned)(D / 4) * 0x9E3779B1u + qb.seed;
         const int rslot = sa == 0 ? RR_RING - 1 : sa - 1;   // (i + RQ + RR_RING - 1) % RR_RING
@@ -557,7 +569,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
             constexpr int every = 2 * NBA;
             const int pc = (nb - NBB) * 8 + c;
             if (pc % every == 0) rows_piece(rslot, qr, pc / every);
-            r_update_piece<MODE, WD, 0>(c, nb, aa[nb - NBB], wq[nb - NBB], t, hs, outw, bl, qb, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, nok, nullptr, 0);
+            r_update_piece<MODE, WD, 0>(c, nb, aa[nb - NBB], wq[nb - NBB], t, hs, outw, knew, bl, qb, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, nok, nullptr, 0);
           }
         if (NBB == 4) rows_pieces(rslot, qr);
       }
@@ -661,7 +673,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     floatx4 aa[2][3];       // A^T of the block in progress and of the one being rounded
     unsigned wq[2][3];      // their old weights
     float t[3][4];
-    unsigned hs[3], outw[3];
+    unsigned hs[3], outw[3], knew[6];
     RKahanBlock kb[2] = {};   // compensation terms of the block in progress and of the one being rounded
     // (this loop must be unrolled completely: its register arrays are indexed by k.  The variants with the Philox
     // recipe or a compensated head exceed the compiler's default size limit for "#pragma unroll" and are compiled in a
@@ -706,13 +718,13 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
       }
       if (k >= 8 && k < NALT) {
         const int o = (k >> 3) - 1;
-        r_update_piece<MODE, WD, KT>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
+        r_update_piece<MODE, WD, KT>(k & 7, o, aa[o & 1], wq[o & 1], t, hs, outw, knew, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
       } else if (k >= NALT && NBB > 0) {
         constexpr int per = NBB == 4 ? 8 : 8 / (16 - 4 * NBB);   // pieces per trailing step
         const int o = NBB - 1;
 #pragma unroll
         for (int c = (k - NALT) * per; c < (k - NALT + 1) * per && c < 8; c++)
-          r_update_piece<MODE, WD, KT>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
+          r_update_piece<MODE, WD, KT>(c, o, aa[o & 1], wq[o & 1], t, hs, outw, knew, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[o & 1], p.kahan, p.num_head);
       }
       if (k < NALT && (k & 1) == 0) {
         const int o = k >> 3, ks = (k & 7) >> 1;
@@ -729,7 +741,7 @@ __global__ __launch_bounds__(QNT, 1) void fp8_step_role_kernel(const QuadParams 
     }
     if (NBB == 4) {
 #pragma unroll
-      for (int c = 0; c < 8; c++) r_update_piece<MODE, WD, KT>(c, 3, aa[1], wq[1], t, hs, outw, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[1], p.kahan, p.num_head);
+      for (int c = 0; c < 8; c++) r_update_piece<MODE, WD, KT>(c, 3, aa[1], wq[1], t, hs, outw, knew, bl, q, hash_tile, p.lr_eff, p.wd_eff, l16, lds, oimg, kb[1], p.kahan, p.num_head);
     }
     q_p = q;
     q_n = q_desc_full(cdesc, tile_at(i + 1));
